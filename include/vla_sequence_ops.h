@@ -139,7 +139,8 @@ int vla_seq_window_attention_tiles(void* out, int64_t out_stride, const void* q,
  *   y given:        y' = y + y_bias (null: none);
  *                   x += y' / sqrt(mean(y'^2) + eps) * post_weight * layer_scale (layer_scale null: 1)
  *   add_row given:  x += add_row
- *   out given:      out = out_dtype(x / sqrt(mean(x^2) + eps) * pre_weight)
+ *   out given:      out = out_dtype(x / sqrt(mean(x^2) + eps) * pre_weight), or out_dtype(x) when
+ *                   pre_weight is null
  * y is `y_dtype` rows of `width` values with stride y_stride; weights, layer_scale, add_row fp32
  * [width].  All of it fp32. */
 int vla_seq_residual_norms(float* x, const void* y, int64_t y_stride, int y_dtype,
@@ -231,14 +232,15 @@ int vla_seq_mingru_scan(void* out, int64_t out_stride, const void* zp, int64_t z
 
 /* ---- mixture of experts in the activation dtype -------------------------------------------------- */
 
-/* Router of one token over `routed` experts (at most 512): z = router h in fp32 (router fp32
- * [routed, width]), s = softmax(z), the `top` largest s + correction (null: s) are chosen, weights
- * = their s / (sum + 1e-20).  experts int32 / weights fp32 [T, top].  shared_gate given:
+/* Router of one token over `routed` experts (at most 512): z = router h + bias in fp32 (router
+ * fp32 [routed, width], bias fp32 [routed] or null), s = softmax(z), the `top` largest s +
+ * correction (null: s) are chosen, weights = their s / (sum + 1e-20) -- without a correction that
+ * is the softmax over the chosen logits.  experts int32 / weights fp32 [T, top].  shared_gate given:
  * shared_gate[t] = sigmoid(shared_gate_weight . h), shared_gate_weight fp32 [width].  logits given
  * (fp32 rows of routed (+ 1 with a shared gate, its logit last) values, stride logits_stride): the
  * products are the caller's and h, router, shared_gate_weight are not read. */
 int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router, const float* logits,
-                      int64_t logits_stride, const float* correction,
+                      int64_t logits_stride, const float* bias, const float* correction,
                       const float* shared_gate_weight, int* experts, float* weights,
                       float* shared_gate, int num_tokens, int width, int routed, int top, int dtype,
                       void* stream);
@@ -271,6 +273,107 @@ int vla_seq_moe_combine(float* out, const float* y, const int* pair_row, const f
                         const void* h, int64_t h_stride, const float* shared_y,
                         const float* shared_gate, int num_tokens, int width, int top, int dtype,
                         void* stream);
+
+/* ---- layers that norm the stream itself after every sublayer --------------------------------------- */
+
+/* x (fp32 [T, width], in place) <- (alpha x + y) / sqrt(mean((alpha x + y)^2) + eps) * weight;
+ * out (null: none) = out_dtype(new x).  y: `y_dtype` rows of `width` values with stride y_stride. */
+int vla_seq_post_norm(float* x, float alpha, const void* y, int64_t y_stride, int y_dtype,
+                      const float* weight, float eps, void* out, int out_dtype, int num_tokens,
+                      int width, void* stream);
+
+/* out = out_dtype(in / sqrt(mean(in^2) + eps) * weight) per row of n values; fp32 arithmetic. */
+int vla_seq_rms_norm_rows(void* out, int64_t out_stride, int out_dtype, const void* in,
+                          int64_t in_stride, int in_dtype, const float* weight, float eps,
+                          int num_tokens, int n, void* stream);
+
+/* Causal convolution over time on each channel:
+ *   out[t] = out_dtype(act(bias + sum_j weight[:, j] u[t - taps + 1 + j])),  zeros before a
+ * sequence's start; weight fp32 [channels, taps], bias fp32 [channels] or null, act a VLA_ACT_*
+ * code.  The last taps - 1 inputs of a sequence live in state fp32 [num_slots, taps - 1, channels]
+ * (oldest first): rows of earlier steps are read from there, and the step leaves its own last
+ * inputs there.  taps <= 32. */
+int vla_seq_short_conv(void* out, int64_t out_stride, int out_dtype, const void* u, int64_t u_stride,
+                       int u_dtype, const float* weight, const float* bias, float* state,
+                       const int* query_start_loc, const int* context_lens, const int* state_slots,
+                       const int* token_seq, int num_tokens, int num_seqs, int num_slots,
+                       int channels, int taps, int act, void* stream);
+
+/* out[t, c] = out_dtype(act(gate[t, c]) * table[ids[t], first_col + c]), c < features. */
+int vla_seq_gated_act_lookup(void* out, int64_t out_stride, int out_dtype, const void* gate,
+                             int64_t gate_stride, int gate_dtype, const void* table,
+                             int64_t table_stride, int table_dtype, const int64_t* ids, int rows,
+                             int first_col, int num_tokens, int features, int act, void* stream);
+
+/* out[t, :] (fp32) = table[ids[t], :] * scale. */
+int vla_seq_embed_scaled(float* out, const void* table, const int64_t* ids, float scale,
+                         int num_tokens, int width, int vocab, int dtype, void* stream);
+
+/* z <- cap * tanh(z / cap) over n fp32 values. */
+int vla_seq_softcap(float* z, int64_t n, float cap, void* stream);
+
+/* ---- gated delta rule ----------------------------------------------------------------------------- */
+
+/* Per head, with a state S fp32 [dim, vdim] per sequence (stored [num_slots, heads, vdim, dim]):
+ *   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+ * k, q of the head's key head (heads / kv_heads value heads share one) divided by
+ * sqrt(sum of squares + 1e-6), q also times dim^-1/2; beta = sigmoid(beta row); g = exp(-exp(a_log)
+ * softplus(dt row + dt_bias)); out = out_dtype(o / sqrt(mean_v(o^2) + eps) * norm_weight *
+ * silu(gate)).  q, k [T, kv_heads * dim], v, gate, out [T, heads * vdim], beta, dt [T, heads]:
+ * rows with their own strides, inputs fp32 (in_dtype VLA_F32).  A sequence with context 0 starts
+ * from zero.  vdim * (dim / 64 rounded up to a power of two) <= 1024. */
+int vla_seq_delta_rule_scan(void* out, int64_t out_stride, int out_dtype, const void* q,
+                            int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                            int64_t v_stride, const void* gate, int64_t gate_stride,
+                            const void* beta, int64_t beta_stride, const void* dt, int64_t dt_stride,
+                            int in_dtype, const float* a_log, const float* dt_bias,
+                            const float* norm_weight, float* state, const int* query_start_loc,
+                            const int* context_lens, const int* state_slots, int num_seqs,
+                            int num_slots, int heads, int kv_heads, int dim, int vdim, float eps,
+                            void* stream);
+
+/* ---- real-gated linear recurrent unit ------------------------------------------------------------- */
+
+/* S_t = a S_(t-1) + sqrt(1 - a^2) sigmoid(i) u per channel, a = exp(-rate sigmoid(r));
+ * out = out_dtype(S_t * gelu_tanh(y)).  u, y fp32 rows of `channels` values with their own
+ * strides; the gates' rows r, i come in blocks of gate_block channels, channel c of token t at
+ * t * stride + (c / gate_block) * gate_block_stride + c % gate_block (the blocks of a batched
+ * product; plain rows: gate_block = channels); rate fp32 [channels], state fp32 [num_slots,
+ * channels]; scratch as for
+ * vla_seq_mingru_scan (vla_seq_mingru_scratch_floats values). */
+int vla_seq_rglru_scan(void* out, int64_t out_stride, int out_dtype, const float* r, int64_t r_stride,
+                       const float* i, int64_t i_stride, int gate_block, int64_t gate_block_stride,
+                       const float* u, int64_t u_stride,
+                       const float* y, int64_t y_stride, const float* rate, float* state,
+                       const int* query_start_loc, const int* context_lens, const int* state_slots,
+                       int num_seqs, int num_slots, int max_query_len, int channels, float* scratch,
+                       int64_t scratch_floats, void* stream);
+
+/* ---- attention over a cached latent ----------------------------------------------------------------- */
+
+/* cache [num_blocks, block_size, rank + rot] (`dtype`): per token the normed latent and the rotated
+ * key part every head shares.  Rotates the rot_dims first elements of every head's rotated query
+ * part in place (head h's part starts at q + t q_stride + h q_head_stride + q_first; interleaved
+ * pairs (2i, 2i + 1) turn by positions[t] * inv_freq[i], sine and cosine times `magnitude`) and
+ * writes the rows [kv[:rank] / sqrt(mean^2 + eps) * norm_weight | kv[rank:] rotated the same way].
+ * slot_mapping < 0 skips the cache. */
+int vla_seq_latent_rotary_write(void* q, int64_t q_stride, int q_head_stride, int q_first,
+                                const void* kv, int64_t kv_stride, const float* norm_weight,
+                                float eps, void* cache, const int64_t* positions,
+                                const int64_t* slot_mapping, const float* inv_freq, float magnitude,
+                                int num_tokens, int heads, int rank, int rot, int rot_dims,
+                                int block_size, int num_blocks, int dtype, void* stream);
+
+/* out[t, h, :rank] = sum_j p_j c_j over the keys j <= position of the row's sequence, p = softmax
+ * of (q_lat[t, h] . c_j + q_rot[t, h] . k_rot_j) * scale; q_lat, q_rot and out are addressed by a
+ * token stride and a head stride each.  Any dtype, rank and rot up to 1024. */
+int vla_seq_latent_attention(void* out, int64_t out_token_stride, int64_t out_head_stride,
+                             const void* q_lat, int64_t lat_token_stride, int64_t lat_head_stride,
+                             const void* q_rot, int64_t rot_token_stride, int64_t rot_head_stride,
+                             const void* cache, const int* block_tables, int max_blocks,
+                             const int* token_seq, const int64_t* positions, int num_tokens,
+                             int heads, int rank, int rot, int block_size, int num_blocks,
+                             float scale, int dtype, void* stream);
 
 /* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);
  * scan 0 = per shape, 1 = token by token. */

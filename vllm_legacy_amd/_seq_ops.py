@@ -267,7 +267,7 @@ def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, y_bias: Op
                    out: Optional[torch.Tensor] = None, pre_weight: Optional[torch.Tensor] = None,
                    eps: float = 1e-5) -> None:
     """x (fp32 [T, W], in place) += y' / rms(y') * post_weight * layer_scale with y' = y + y_bias;
-    x += add_row; out = x / rms(x) * pre_weight.  Each part is optional."""
+    x += add_row; out = x / rms(x) * pre_weight (pre_weight None: out = x).  Each part is optional."""
     _gpu(x, y, y_bias, post_weight, layer_scale, add_row, out, pre_weight)
     T, W = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
@@ -276,7 +276,7 @@ def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, y_bias: Op
     if y is not None:
         assert y.shape == x.shape and post_weight is not None
     if out is not None:
-        assert out.shape == x.shape and out.is_contiguous() and pre_weight is not None
+        assert out.shape == x.shape and out.is_contiguous()
     with torch.cuda.device(x.device):
         seq_check(_lib.seq_lib().vla_seq_residual_norms(
             x.data_ptr(), _p(y), 0 if y is None else _rows(y, W), _lib.F32 if y is None else _dt(y.dtype),
@@ -447,13 +447,15 @@ def mingru_scan(out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor],
-              shared_gate_weight: Optional[torch.Tensor], top: int, logits: Optional[torch.Tensor] = None):
+              shared_gate_weight: Optional[torch.Tensor], top: int, logits: Optional[torch.Tensor] = None,
+              bias: Optional[torch.Tensor] = None):
     """-> experts int32 [T, top], weights fp32 [T, top], shared gate fp32 [T] or None.  logits
     (fp32 [T, routed (+ 1, the shared gate's last)]): the router products, when the caller formed
     them as one matrix product."""
-    _gpu(h, router, correction, shared_gate_weight, logits)
+    _gpu(h, router, correction, shared_gate_weight, logits, bias)
     T, W = h.shape
     N = router.shape[0]
+    assert bias is None or (bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous())
     assert router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == W
     assert correction is None or (correction.dtype == torch.float32 and correction.numel() == N)
     assert shared_gate_weight is None or (shared_gate_weight.dtype == torch.float32 and shared_gate_weight.numel() == W)
@@ -466,7 +468,7 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.
     with torch.cuda.device(h.device):
         seq_check(_lib.seq_lib().vla_seq_moe_route(
             h.data_ptr(), _rows(h, W), router.data_ptr(), _p(logits), 0 if logits is None else logits.shape[1],
-            _p(correction), _p(shared_gate_weight), experts.data_ptr(), weights.data_ptr(), _p(sg), T, W, N,
+            _p(bias), _p(correction), _p(shared_gate_weight), experts.data_ptr(), weights.data_ptr(), _p(sg), T, W, N,
             int(top), _dt(h.dtype), _stream(h.device)), "moe_route")
     return experts, weights, sg
 
@@ -524,3 +526,200 @@ def moe_combine(out: torch.Tensor, y: torch.Tensor, pair_row: torch.Tensor, weig
         seq_check(_lib.seq_lib().vla_seq_moe_combine(
             out.data_ptr(), y.data_ptr(), pair_row.data_ptr(), weights.data_ptr(), h.data_ptr(), _rows(h, W),
             _p(shared_y), _p(shared_gate), T, W, top, _dt(h.dtype), _stream(h.device)), "moe_combine")
+
+
+# ---------------------------------------------------------------- layers that norm the stream itself
+def post_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, alpha: float, eps: float,
+              out: Optional[torch.Tensor] = None) -> None:
+    """x (fp32 [T, W], in place) <- (alpha x + y) / rms(alpha x + y) * weight; out = the new x in
+    out's dtype."""
+    _gpu(x, y, weight, out)
+    T, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and y.shape == x.shape
+    assert weight.dtype == torch.float32 and weight.numel() == W and weight.is_contiguous()
+    assert out is None or (out.shape == x.shape and out.is_contiguous())
+    with torch.cuda.device(x.device):
+        seq_check(_lib.seq_lib().vla_seq_post_norm(
+            x.data_ptr(), float(alpha), y.data_ptr(), _rows(y, W), _dt(y.dtype), weight.data_ptr(), float(eps),
+            _p(out), _lib.F32 if out is None else _dt(out.dtype), T, W, _stream(x.device)), "post_norm")
+
+
+def rms_norm_rows(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """out = x / rms(x) * weight per row; [T, n] views with free row strides, any dtypes."""
+    _gpu(out, x, weight)
+    T, n = x.shape
+    assert out.shape == x.shape and weight.dtype == torch.float32 and weight.numel() == n and weight.is_contiguous()
+    with torch.cuda.device(x.device):
+        seq_check(_lib.seq_lib().vla_seq_rms_norm_rows(
+            out.data_ptr(), _rows(out, n), _dt(out.dtype), x.data_ptr(), _rows(x, n), _dt(x.dtype),
+            weight.data_ptr(), float(eps), T, n, _stream(x.device)), "rms_norm_rows")
+
+
+def short_conv(out: torch.Tensor, u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+               state: Optional[torch.Tensor], query_start_loc: torch.Tensor, context_lens: torch.Tensor,
+               state_slots: torch.Tensor, token_seq: torch.Tensor, act: str = "none") -> None:
+    """out = act(bias + conv(u)) along time per channel; out, u [T, C] views with free row strides;
+    weight fp32 [C, taps]; state fp32 [slots, taps - 1, C] holds every sequence's last inputs and is
+    brought up to date."""
+    _gpu(out, u, weight, bias, state, query_start_loc, context_lens, state_slots, token_seq)
+    T, Cn = u.shape
+    taps = weight.shape[1]
+    B = context_lens.numel()
+    assert out.shape == u.shape
+    assert weight.dtype == torch.float32 and weight.is_contiguous() and weight.shape[0] == Cn
+    assert bias is None or (bias.dtype == torch.float32 and bias.numel() == Cn and bias.is_contiguous())
+    slots = 0
+    if taps > 1:
+        assert state is not None and state.dtype == torch.float32 and state.is_contiguous()
+        assert state.shape[1:] == (taps - 1, Cn)
+        slots = state.shape[0]
+    for t in (query_start_loc, context_lens, state_slots, token_seq):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert query_start_loc.numel() == B + 1 and state_slots.numel() == B and token_seq.numel() == T
+    with torch.cuda.device(u.device):
+        seq_check(_lib.seq_lib().vla_seq_short_conv(
+            out.data_ptr(), _rows(out, Cn), _dt(out.dtype), u.data_ptr(), _rows(u, Cn), _dt(u.dtype),
+            weight.data_ptr(), _p(bias), _p(state if taps > 1 else None), query_start_loc.data_ptr(),
+            context_lens.data_ptr(), state_slots.data_ptr(), token_seq.data_ptr(), T, B, slots, Cn, taps, ACT[act],
+            _stream(u.device)), "short_conv")
+
+
+def gated_act_lookup(out: torch.Tensor, gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor,
+                     first_col: int, act: str) -> None:
+    """out[t] = act(gate[t]) * table[ids[t], first_col : first_col + F]; out, gate [T, F]."""
+    _gpu(out, gate, table, ids)
+    T, F = gate.shape
+    assert out.shape == gate.shape and table.dim() == 2 and table.stride(1) == 1
+    assert ids.dtype == torch.int64 and ids.numel() == T and ids.is_contiguous()
+    assert 0 <= first_col and first_col + F <= table.shape[1]
+    with torch.cuda.device(gate.device):
+        seq_check(_lib.seq_lib().vla_seq_gated_act_lookup(
+            out.data_ptr(), _rows(out, F), _dt(out.dtype), gate.data_ptr(), _rows(gate, F), _dt(gate.dtype),
+            table.data_ptr(), table.stride(0), _dt(table.dtype), ids.data_ptr(), table.shape[0], int(first_col), T, F,
+            ACT[act], _stream(gate.device)), "gated_act_lookup")
+
+
+def embed_scaled(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float) -> None:
+    _gpu(out, table, ids)
+    T, W = out.shape
+    assert out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous() and table.shape[1] == W
+    assert ids.dtype == torch.int64 and ids.numel() == T and ids.is_contiguous()
+    with torch.cuda.device(out.device):
+        seq_check(_lib.seq_lib().vla_seq_embed_scaled(
+            out.data_ptr(), table.data_ptr(), ids.data_ptr(), float(scale), T, W, table.shape[0], _dt(table.dtype),
+            _stream(out.device)), "embed_scaled")
+
+
+def softcap(z: torch.Tensor, cap: float) -> None:
+    """z (fp32, in place) <- cap * tanh(z / cap)."""
+    _gpu(z)
+    assert z.dtype == torch.float32 and z.is_contiguous()
+    with torch.cuda.device(z.device):
+        seq_check(_lib.seq_lib().vla_seq_softcap(z.data_ptr(), z.numel(), float(cap), _stream(z.device)), "softcap")
+
+
+def delta_rule_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
+                    beta: torch.Tensor, dt: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                    norm_weight: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor,
+                    context_lens: torch.Tensor, state_slots: torch.Tensor, kv_heads: int, eps: float) -> None:
+    """out [T, H*V]; q, k fp32 [T, G*D]; v, gate fp32 [T, H*V]; beta, dt fp32 [T, H] (views with free
+    row strides); a_log, dt_bias fp32 [H]; norm_weight fp32 [V]; state fp32 [slots, H, V, D]."""
+    _gpu(out, q, k, v, gate, beta, dt, a_log, dt_bias, norm_weight, state, query_start_loc, context_lens, state_slots)
+    slots, H, V, D = state.shape
+    B = context_lens.numel()
+    assert state.dtype == torch.float32 and state.is_contiguous()
+    for t in (q, k, v, gate, beta, dt):
+        assert t.dtype == torch.float32
+    for t in (a_log, dt_bias, norm_weight):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    assert a_log.numel() == H and dt_bias.numel() == H and norm_weight.numel() == V
+    for t in (query_start_loc, context_lens, state_slots):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert query_start_loc.numel() == B + 1 and state_slots.numel() == B
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_delta_rule_scan(
+            out.data_ptr(), _rows(out, H * V), _dt(out.dtype), q.data_ptr(), _rows(q, kv_heads * D), k.data_ptr(),
+            _rows(k, kv_heads * D), v.data_ptr(), _rows(v, H * V), gate.data_ptr(), _rows(gate, H * V),
+            beta.data_ptr(), _rows(beta, H), dt.data_ptr(), _rows(dt, H), _lib.F32, a_log.data_ptr(),
+            dt_bias.data_ptr(), norm_weight.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
+            context_lens.data_ptr(), state_slots.data_ptr(), B, slots, H, int(kv_heads), D, V, float(eps),
+            _stream(q.device)), "delta_rule_scan")
+
+
+def rglru_scan(out: torch.Tensor, gates: torch.Tensor, u: torch.Tensor, y: torch.Tensor,
+               rate: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
+               state_slots: torch.Tensor, max_query_len: int) -> None:
+    """out [T, R]; gates fp32 [blocks, T, 2 * R / blocks] contiguous (per block: the recurrence
+    gate's products, then the input gate's); u, y fp32 [T, R] views; rate fp32 [R]; state fp32
+    [slots, R]."""
+    _gpu(out, gates, u, y, rate, state, query_start_loc, context_lens, state_slots)
+    T, R = u.shape
+    B = context_lens.numel()
+    blocks = gates.shape[0]
+    bw = R // blocks
+    assert gates.dtype == torch.float32 and gates.is_contiguous() and gates.shape == (blocks, T, 2 * bw)
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == R
+    for t in (u, y):
+        assert t.dtype == torch.float32 and t.shape == (T, R)
+    assert rate.dtype == torch.float32 and rate.numel() == R and rate.is_contiguous()
+    for t in (query_start_loc, context_lens, state_slots):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    L = _lib.seq_lib()
+    need = L.vla_seq_mingru_scratch_floats(B, int(max_query_len), R)
+    scratch = torch.empty(need, dtype=torch.float32, device=u.device) if need else None
+    with torch.cuda.device(u.device):
+        seq_check(L.vla_seq_rglru_scan(
+            out.data_ptr(), _rows(out, R), _dt(out.dtype), gates.data_ptr(), 2 * bw, gates.data_ptr() + 4 * bw,
+            2 * bw, bw, T * 2 * bw, u.data_ptr(), _rows(u, R), y.data_ptr(), _rows(y, R), rate.data_ptr(),
+            state.data_ptr(), query_start_loc.data_ptr(), context_lens.data_ptr(), state_slots.data_ptr(), B,
+            state.shape[0], int(max_query_len), R, _p(scratch), need, _stream(u.device)), "rglru_scan")
+
+
+def latent_rotary_write(q: torch.Tensor, q_head_stride: int, q_first: int, heads: int, kv: torch.Tensor,
+                        norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, positions: torch.Tensor,
+                        slot_mapping: torch.Tensor, inv_freq: Optional[torch.Tensor], magnitude: float,
+                        rot_dims: int) -> None:
+    """q [T, >= heads * q_head_stride]: the rotated part of head h starts at column h * q_head_stride +
+    q_first; kv [T, rank + rot]; cache [NB, BS, rank + rot]."""
+    _gpu(q, kv, norm_weight, cache, positions, slot_mapping, inv_freq)
+    NB, BS, width = cache.shape
+    rank = norm_weight.numel()
+    rot = width - rank
+    T = q.shape[0]
+    assert cache.is_contiguous() and q.dtype == kv.dtype == cache.dtype and q.stride(1) == 1
+    assert kv.shape == (T, width) and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous()
+    assert (heads - 1) * q_head_stride + q_first + rot <= q.shape[1]
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() == T and slot_mapping.is_contiguous()
+    if rot_dims:
+        assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2 and inv_freq.is_contiguous()
+    with torch.cuda.device(q.device):
+        seq_check(_lib.seq_lib().vla_seq_latent_rotary_write(
+            q.data_ptr(), q.stride(0) if T > 1 else q.shape[1], int(q_head_stride), int(q_first), kv.data_ptr(),
+            _rows(kv, width), norm_weight.data_ptr(), float(eps), cache.data_ptr(), positions.data_ptr(),
+            slot_mapping.data_ptr(), _p(inv_freq), float(magnitude), T, int(heads), rank, rot, int(rot_dims), BS, NB,
+            _dt(q.dtype), _stream(q.device)), "latent_rotary_write")
+
+
+def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
+                     block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
+                     scale: float) -> None:
+    """out, q_lat [T, H, rank] and q_rot [T, H, rot] views (any token / head strides, unit stride
+    along the last axis); cache [NB, BS, rank + rot]."""
+    _gpu(out, q_lat, q_rot, cache, block_tables, token_seq, positions)
+    NB, BS, width = cache.shape
+    T, H, rank = q_lat.shape
+    rot = width - rank
+    assert out.shape == q_lat.shape and q_rot.shape == (T, H, rot) and cache.is_contiguous()
+    assert out.dtype == q_lat.dtype == q_rot.dtype == cache.dtype
+    for t in (out, q_lat, q_rot):
+        assert t.stride(2) == 1 or t.shape[2] == 1
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    assert token_seq.dtype == torch.int32 and token_seq.numel() == T and token_seq.is_contiguous()
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    with torch.cuda.device(q_lat.device):
+        seq_check(_lib.seq_lib().vla_seq_latent_attention(
+            out.data_ptr(), out.stride(0), out.stride(1), q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1),
+            q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], token_seq.data_ptr(), positions.data_ptr(), T, H, rank, rot, BS, NB, float(scale),
+            _dt(q_lat.dtype), _stream(q_lat.device)), "latent_attention")

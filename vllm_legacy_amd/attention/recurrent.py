@@ -151,3 +151,81 @@ class MinGRURecurrence(nn.Module):
         ops.mingru_scan(out, zp, up, gp, state, batch.query_start_loc, batch.context_lens, batch.state_slots,
                         batch.max_query_len)
         return out
+
+
+class GatedDeltaRule(nn.Module):
+    """Gated delta rule with per-sequence state slots.  Per head, on a state S [dim, vdim]:
+    S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q -- the read-out sees the token's
+    own write.  k and q are unit vectors per key head (q also times dim^-1/2), `heads / kv_heads`
+    value heads share a key head, beta = sigmoid(b), g = exp(-exp(A_log) softplus(dt + dt_bias)),
+    and o leaves RMS-normed over vdim, weighted (one weight vector for all heads) and times
+    silu(gate).  All inputs are fp32 rows (the caller's projections and short convolutions leave
+    them so); the state is fp32 [num_slots, heads, vdim, dim] and a sequence whose context length
+    is 0 starts from zero whatever its slot held (csrc/seq_delta_rule.hip)."""
+
+    def __init__(self, heads: int, kv_heads: int, dim: int, vdim: int, eps: float, device=None) -> None:
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.heads, self.kv_heads, self.dim, self.vdim, self.eps = heads, kv_heads, dim, vdim, float(eps)
+
+        def par(n, fill=0.0):
+            return nn.Parameter(torch.full((n, ), fill, dtype=torch.float32, device=device), requires_grad=False)
+
+        self.a_log, self.dt_bias, self.norm_weight = par(heads), par(heads), par(vdim, 1.0)
+
+    @staticmethod
+    def get_state_shape(num_slots: int, heads: int, dim: int, vdim: int) -> Tuple[int, ...]:
+        return (num_slots, heads, vdim, dim)
+
+    def forward(self, out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
+                beta: torch.Tensor, dt: torch.Tensor, state: torch.Tensor, batch: SequenceBatch) -> torch.Tensor:
+        """q, k [T, G*D]; v, gate, out [T, H*V]; beta, dt [T, H]: views with free row strides."""
+        ops.delta_rule_scan(out, q, k, v, gate, beta, dt, self.a_log.data, self.dt_bias.data, self.norm_weight.data,
+                            state, batch.query_start_loc, batch.context_lens, batch.state_slots, self.kv_heads,
+                            self.eps)
+        return out
+
+
+class RealGatedLRU(nn.Module):
+    """Real-gated linear recurrent unit: per channel S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with
+    a_t = exp(-c r_t softplus(lam)), r = sigmoid(W_a u + b_a), i = sigmoid(W_i u + b_i), where W_a and
+    W_i are block-diagonal (`blocks` square blocks [out, in]); the output is S_t * gelu_tanh(y_t).
+    u and y are fp32 rows; the gates' products are fp32 batched matrix products; the state is fp32
+    [num_slots, channels] and a sequence whose context length is 0 starts from zero.  Long runs of
+    rows are walked in pieces at the same time (csrc/seq_gated_recurrence.hip)."""
+
+    def __init__(self, channels: int, blocks: int, c: float = 8.0, device=None) -> None:
+        super().__init__()
+        assert channels % blocks == 0
+        self.channels, self.blocks, self.c = channels, blocks, float(c)
+        bw = channels // blocks
+        # both gates' blocks side by side: [blocks, in, 2 * out] (recurrence gate | input gate)
+        self.gate_weight = nn.Parameter(torch.zeros((blocks, bw, 2 * bw), dtype=torch.float32, device=device),
+                                        requires_grad=False)
+        self.gate_bias = nn.Parameter(torch.zeros((blocks, 1, 2 * bw), dtype=torch.float32, device=device),
+                                      requires_grad=False)
+        self.rate = nn.Parameter(torch.zeros(channels, dtype=torch.float32, device=device), requires_grad=False)
+
+    def set_weights(self, ra, ra_b, ri, ri_b, lam) -> None:
+        """ra, ri [blocks, out, in]; ra_b, ri_b [blocks, out]; lam [channels]."""
+        dev = self.rate.device
+        w = torch.cat([ra.float().transpose(1, 2), ri.float().transpose(1, 2)], 2)
+        b = torch.cat([ra_b.float(), ri_b.float()], 1)[:, None, :]
+        self.gate_weight.data = w.to(dev).contiguous()
+        self.gate_bias.data = b.to(dev).contiguous()
+        self.rate.data = (self.c * torch.nn.functional.softplus(lam.float())).to(dev).contiguous()
+
+    @staticmethod
+    def get_state_shape(num_slots: int, channels: int) -> Tuple[int, ...]:
+        return (num_slots, channels)
+
+    def forward(self, out: torch.Tensor, u: torch.Tensor, y: torch.Tensor, state: torch.Tensor,
+                batch: SequenceBatch) -> torch.Tensor:
+        """u fp32 [T, R] contiguous (the recurrent branch after its convolution), y fp32 [T, R] view (the
+        other branch before its activation), out [T, R]."""
+        T, R = u.shape
+        B, bw = self.blocks, R // self.blocks
+        gates = torch.baddbmm(self.gate_bias.data, u.view(T, B, bw).transpose(0, 1), self.gate_weight.data)
+        ops.rglru_scan(out, gates, u, y, self.rate.data, state, batch.query_start_loc, batch.context_lens,
+                       batch.state_slots, batch.max_query_len)
+        return out

@@ -72,6 +72,16 @@ __global__ __launch_bounds__(kThreads) void residual_norms_kernel(
                                               (y_bias != nullptr ? y_bias[c] : 0.f)
                                         : 0.f);
   if (out == nullptr) return;
+  if (pre_w == nullptr) {           // no norm ahead of the reader: the stream's row as it is
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int c = threadIdx.x + i * kThreads;
+      if (c < width) out[base + c] = SO::from_f32(keep[i]);
+    }
+    for (int c = threadIdx.x + kKeep * kThreads; c < width; c += kThreads)
+      out[base + c] = SO::from_f32(x[base + c]);
+    return;
+  }
   ss = block_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)width + eps);
 #pragma unroll
@@ -218,8 +228,7 @@ extern "C" int vla_seq_residual_norms(float* x, const void* y, int64_t y_stride,
                                       float eps, int num_tokens, int width, int out_dtype,
                                       void* stream) {
   if (num_tokens == 0) return VLA_OK;
-  if (!x || num_tokens < 0 || width <= 0 || (y && (!post_weight || y_stride < width)) ||
-      (out && !pre_weight))
+  if (!x || num_tokens < 0 || width <= 0 || (y && (!post_weight || y_stride < width)))
     return VLA_ERR_ARG;
   return with_two_dtypes(y ? y_dtype : VLA_F32, out ? out_dtype : VLA_F32, [&](auto sy, auto so) {
     using SY = decltype(sy);

@@ -1,6 +1,6 @@
 // Mixture-of-experts feed-forward in the activation dtype (no quantization), routed on the device
 // without a host synchronisation:
-//   moe_route      per token: router logits in fp32, softmax over all experts, choice by score plus
+//   moe_route      per token: router logits in fp32 (plus a bias), softmax over all experts, choice by score plus
 //                  a per-expert correction, weights = chosen scores renormalized; also the sigmoid
 //                  gate of a shared expert
 //   moe_plan       groups the (token, choice) pairs by expert into row tiles of kTile rows (groups
@@ -40,7 +40,8 @@ __device__ __forceinline__ float act_apply(float z, int act) {
 template <class S>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     const typename S::T* __restrict__ h, int64_t h_stride, const float* __restrict__ router,
-    const float* __restrict__ logits, int64_t logits_stride, const float* __restrict__ correction,
+    const float* __restrict__ logits, int64_t logits_stride, const float* __restrict__ bias,
+    const float* __restrict__ correction,
     const float* __restrict__ shared_gate_w, int* __restrict__ experts, float* __restrict__ weights,
     float* __restrict__ shared_gate, int width, int routed, int top) {
   __shared__ float z[kMaxRouted + 1];
@@ -48,7 +49,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   const bool gated = shared_gate != nullptr;
   const int rows = routed + (gated ? 1 : 0);
   if (logits != nullptr) {
-    for (int n = threadIdx.x; n < rows; n += 256) z[n] = logits[(int64_t)t * logits_stride + n];
+    for (int n = threadIdx.x; n < rows; n += 256)
+      z[n] = logits[(int64_t)t * logits_stride + n] + (bias != nullptr && n < routed ? bias[n] : 0.f);
   } else {
     const typename S::T* hr = h + (int64_t)t * h_stride;
     for (int n = w; n < rows; n += 4) {
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
       float dot = 0.f;
       for (int c = lane; c < width; c += kWave) dot += wr[c] * S::to_f32(hr[c]);
       dot = wave_sum(dot);
-      if (lane == 0) z[n] = dot;
+      if (lane == 0) z[n] = dot + (bias != nullptr && n < routed ? bias[n] : 0.f);
     }
   }
   __syncthreads();
@@ -499,7 +501,7 @@ using namespace vla;
 using namespace vla::seq;
 
 extern "C" int vla_seq_moe_route(const void* h, int64_t h_stride, const float* router,
-                                 const float* logits, int64_t logits_stride,
+                                 const float* logits, int64_t logits_stride, const float* bias,
                                  const float* correction, const float* shared_gate_weight,
                                  int* experts, float* weights, float* shared_gate, int num_tokens,
                                  int width, int routed, int top, int dtype, void* stream) {
@@ -513,7 +515,7 @@ extern "C" int vla_seq_moe_route(const void* h, int64_t h_stride, const float* r
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
     moe_route_kernel<S><<<num_tokens, 256, 0, (hipStream_t)stream>>>(
-        (const typename S::T*)h, h_stride, router, logits, logits_stride, correction,
+        (const typename S::T*)h, h_stride, router, logits, logits_stride, bias, correction,
         shared_gate_weight, experts, weights, shared_gate, width, routed, top);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;

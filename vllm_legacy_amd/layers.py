@@ -162,6 +162,60 @@ class CausalConvMix(nn.Module):
         return out
 
 
+class ShortConv(nn.Module):
+    """act(bias + conv(u)): a causal convolution over time on each channel (weight [channels, taps],
+    the last column weighs the current token, zeros before a sequence's start), with an optional
+    bias and activation.  The last taps - 1 inputs of every sequence live in a state slot
+    [num_slots, taps - 1, channels] (fp32), so a sequence may be cut anywhere.  Input and output are
+    views with free row strides, of any dtype."""
+
+    def __init__(self, channels: int, taps: int, bias: bool = False, act: str = "none", device=None):
+        super().__init__()
+        if act not in seq_ops.ACT:
+            raise ValueError(f"unknown activation {act!r}")
+        self.channels, self.taps, self.act = int(channels), int(taps), act
+        self.weight = nn.Parameter(torch.zeros((channels, taps), dtype=torch.float32, device=device),
+                                   requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(channels, dtype=torch.float32, device=device),
+                                 requires_grad=False) if bias else None
+
+    @staticmethod
+    def get_state_shape(num_slots: int, channels: int, taps: int) -> Tuple[int, ...]:
+        return (num_slots, max(taps - 1, 0), channels)
+
+    def forward(self, out: torch.Tensor, u: torch.Tensor, state: Optional[torch.Tensor], batch) -> torch.Tensor:
+        seq_ops.short_conv(out, u, self.weight.data, None if self.bias is None else self.bias.data,
+                           state if self.taps > 1 else None, batch.query_start_loc, batch.context_lens,
+                           batch.state_slots, batch.token_seq, self.act)
+        return out
+
+
+class TokenGatedInput(nn.Module):
+    """A per-token side input to an fp32 stream: with e the token's row of a side embedding table
+    (columns first_col .. first_col + dim - 1), g = act(W_gate x) * e, y = W_proj g,
+    x += y / rms(y) * weight.  Returns the new stream in the activation dtype as well (what the next
+    sublayer's projections read)."""
+
+    def __init__(self, width: int, dim: int, first_col: int, eps: float, act: str = "gelu_tanh",
+                 dtype=torch.bfloat16, device=None):
+        super().__init__()
+        self.dim, self.first_col, self.eps, self.act, self.dtype = int(dim), int(first_col), float(eps), act, dtype
+        self.gate = nn.Parameter(torch.zeros((dim, width), dtype=dtype, device=device), requires_grad=False)
+        self.proj = nn.Parameter(torch.zeros((width, dim), dtype=dtype, device=device), requires_grad=False)
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        """x fp32 [T, width] (in place), h the same rows in the activation dtype; table the side
+        embedding [vocab, columns]."""
+        gate = torch.mm(h, self.gate.data.t())
+        g = torch.empty_like(gate)
+        seq_ops.gated_act_lookup(g, gate, table, ids, self.first_col, self.act)
+        y = torch.mm(g, self.proj.data.t()) if g.dtype == torch.float32 else \
+            torch.mm(g, self.proj.data.t(), out_dtype=torch.float32)
+        seq_ops.residual_norms(x, y, None, self.weight.data, None, None, h, None, self.eps)
+        return h
+
+
 class GatedActivation(nn.Module):
     """act(gate) * up on the two halves of a merged projection [T, 2 F] (gate | up), or act(z) on
     a plain one; act: relu, relu2 (the square of relu), silu, gelu_tanh."""

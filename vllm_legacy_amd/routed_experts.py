@@ -1,9 +1,10 @@
 """Mixture-of-experts feed-forward in the activation dtype, routed on the device.
 
-Router: z = W_r h in fp32 over all routed experts, s = softmax(z); the `top` experts with the
-largest s + correction are chosen and weighted by their s renormalized to sum 1.  The last
-`identity` routed experts have no weights: their output is the token's input.  An expert is
-W_down act(W_up h).  An optional shared expert of the same form runs for every token, multiplied by
+Router: z = W_r h (+ a bias) in fp32 over all routed experts, s = softmax(z); the `top` experts
+with the largest s + correction are chosen and weighted by their s renormalized to sum 1 (without a
+correction: the softmax over the chosen logits).  The last `identity` routed experts have no
+weights: their output is the token's input.  An expert is W_down act(W_up h), or, `gated`,
+W_down (act(W_gate h) * W_up h).  An optional shared expert of the same form runs for every token, multiplied by
 sigmoid(w_sg . h).  The output is fp32 (the caller norms it and adds it to its stream).
 
 Execution (csrc/seq_moe_kernels.hip): route (the logits of a large step come from one fp32 matrix
@@ -34,7 +35,7 @@ class RoutedExperts(nn.Module):
 
     def __init__(self, width: int, num_experts: int, num_identity: int, top: int, expert_ff: int,
                  shared_ff: int = 0, act: str = "relu2", shared_act: Optional[str] = None,
-                 dtype=torch.bfloat16, device=None) -> None:
+                 dtype=torch.bfloat16, device=None, gated: bool = False, router_bias: bool = False) -> None:
         super().__init__()
         if top > num_experts + num_identity:
             raise ValueError("top exceeds the number of routed experts")
@@ -42,6 +43,7 @@ class RoutedExperts(nn.Module):
         self.expert_ff, self.shared_ff, self.act = expert_ff, shared_ff, act
         self.shared_act = shared_act or act
         self.dtype = dtype
+        self.gated = bool(gated)
         self._router_rows = None
         routed = num_experts + num_identity
 
@@ -50,7 +52,9 @@ class RoutedExperts(nn.Module):
 
         self.router = par((routed, width), torch.float32)
         self.correction = par((routed, ), torch.float32)
-        self.w_up = par((num_experts, expert_ff, width), dtype)
+        self.router_bias = par((routed, ), torch.float32) if router_bias else None
+        # gated experts keep W_gate's rows ahead of W_up's in one matrix per expert
+        self.w_up = par((num_experts, (2 if gated else 1) * expert_ff, width), dtype)
         self.w_down = par((num_experts, width, expert_ff), dtype)
         if shared_ff:
             self.shared_up = par((shared_ff, width), dtype)
@@ -58,7 +62,8 @@ class RoutedExperts(nn.Module):
             self.shared_gate = par((width, ), torch.float32)
 
     def set_weights(self, t: Dict[str, torch.Tensor]) -> None:
-        """t: router, correction (optional), e<i>.up / e<i>.down, shared.up / shared.down / shared.sg."""
+        """t: router, router.b (with a router bias), correction (optional), e<i>.up / e<i>.down
+        (gated: also e<i>.gate), shared.up / shared.down / shared.sg."""
         dev, dt = self.router.device, self.dtype
         routed = self.num_experts + self.num_identity
 
@@ -71,8 +76,14 @@ class RoutedExperts(nn.Module):
         put(self.router, t["router"], "router")
         if "correction" in t:
             put(self.correction, t["correction"].reshape(routed), "correction")
-        if self.num_experts:
+        if self.router_bias is not None:
+            put(self.router_bias, t["router.b"].reshape(routed), "router.b")
+        if self.num_experts and self.gated:
+            put(self.w_up, torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0)
+                                        for e in range(self.num_experts)]).to(dt), "e*.gate | e*.up")
+        elif self.num_experts:
             put(self.w_up, torch.stack([t[f"e{e}.up"] for e in range(self.num_experts)]).to(dt), "e*.up")
+        if self.num_experts:
             put(self.w_down, torch.stack([t[f"e{e}.down"] for e in range(self.num_experts)]).to(dt), "e*.down")
         if self.shared_ff:
             put(self.shared_up, t["shared.up"], "shared.up")
@@ -94,12 +105,18 @@ class RoutedExperts(nn.Module):
             # many tokens: the router rows (and the shared gate's) as one fp32 matrix product
             logits = torch.mm(h if h.dtype == torch.float32 else h.float(), self.router_rows().t())
         experts, weights, sg = ops.moe_route(h, self.router.data, self.correction.data,
-                                             self.shared_gate.data if self.shared_ff else None, self.top, logits)
+                                             self.shared_gate.data if self.shared_ff else None, self.top, logits,
+                                             None if self.router_bias is None else self.router_bias.data)
         if self.num_experts:
             pair_row, row_token, tile_expert = ops.moe_plan(experts, self.num_experts)
             rows = row_token.numel()
             u = torch.empty((rows, self.expert_ff), dtype=h.dtype, device=h.device)
-            ops.grouped_linear(u, h, row_token, self.w_up.data, tile_expert, self.act)
+            if self.gated:
+                both = torch.empty((rows, 2 * self.expert_ff), dtype=h.dtype, device=h.device)
+                ops.grouped_linear(both, h, row_token, self.w_up.data, tile_expert)
+                ops.gated_act(u, both[:, :self.expert_ff], both[:, self.expert_ff:], self.act)
+            else:
+                ops.grouped_linear(u, h, row_token, self.w_up.data, tile_expert, self.act)
             y = torch.empty((rows, self.width), dtype=torch.float32, device=h.device)
             ops.grouped_linear(y, u, None, self.w_down.data, tile_expert)
         else:   # identity experts only
