@@ -47,6 +47,21 @@ def short_convolution(u, w, bias=None):
 
 
 # ----------------------------------------------------------------------------- gated delta rule
+def delta_rule(q, k, v, beta, decay, S=None):
+    """One head: q, k [n, D] (normed already), v [n, V], beta, decay [n].  S <- decay S;
+    u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  Returns o [n, V] (and leaves S updated)."""
+    n, D, V = q.shape[0], q.shape[1], v.shape[1]
+    if S is None:
+        S = torch.zeros(D, V, dtype=F)
+    out = torch.zeros(n, V, dtype=F)
+    for i in range(n):
+        S *= decay[i]
+        u = beta[i] * (v[i] - S.T @ k[i])
+        S += torch.outer(k[i], u)
+        out[i] = S.T @ q[i]
+    return out
+
+
 def delta_mixer(h, t, spec, eps):
     """h [n, W]; t: the mixer's tensors by their short names; spec: heads, kv_heads, dim, vdim."""
     n = h.shape[0]
@@ -62,17 +77,24 @@ def delta_mixer(h, t, spec, eps):
     out = torch.zeros(n, H, V, dtype=F)
     for hh in range(H):
         g = hh // (H // G)
-        S = torch.zeros(D, V, dtype=F)
-        for i in range(n):
-            S = decay[i, hh] * S
-            u = beta[i, hh] * (v[i, hh] - S.T @ k[i, g])
-            S = S + torch.outer(k[i, g], u)
-            out[i, hh] = S.T @ q[i, g]
+        out[:, hh] = delta_rule(q[:, g], k[:, g], v[:, hh], beta[:, hh], decay[:, hh])
     out = out / torch.sqrt((out * out).mean(-1, keepdim=True) + eps) * t["norm"] * gate
     return out.reshape(n, H * V) @ t["o"].T
 
 
 # ----------------------------------------------------------------------------- real-gated LRU
+def rglru_recurrence(u, r, i, lam, S=None):
+    """u, r, i [n, R] (gates after their sigmoid), lam [R]: a = exp(-8 r softplus(lam)),
+    S_t = a S_(t-1) + sqrt(1 - a^2) i u from S = 0.  Returns every S_t."""
+    a = torch.exp(-8.0 * r * softplus(lam))
+    S = torch.zeros(u.shape[1], dtype=F) if S is None else S
+    out = torch.zeros_like(u)
+    for s_ in range(u.shape[0]):
+        S = a[s_] * S + torch.sqrt(1.0 - a[s_]**2) * i[s_] * u[s_]
+        out[s_] = S
+    return out
+
+
 def rglru_mixer(h, t, spec):
     """h [n, W]; spec: width, blocks."""
     n = h.shape[0]
@@ -82,13 +104,7 @@ def rglru_mixer(h, t, spec):
     ub = u.view(n, B, R // B)
     r = torch.sigmoid(torch.einsum("boi,nbi->nbo", t["ra"], ub) + t["ra.b"]).reshape(n, R)
     i = torch.sigmoid(torch.einsum("boi,nbi->nbo", t["ri"], ub) + t["ri.b"]).reshape(n, R)
-    log_a = -8.0 * r * softplus(t["lam"])
-    a = torch.exp(log_a)
-    S = torch.zeros(R, dtype=F)
-    out = torch.zeros(n, R, dtype=F)
-    for s in range(n):
-        S = a[s] * S + torch.sqrt(1.0 - a[s]**2) * i[s] * u[s]
-        out[s] = S
+    out = rglru_recurrence(u, r, i, t["lam"])
     return (out * y) @ t["o"].T
 
 
@@ -214,7 +230,69 @@ def forward(cfg, tensors, tokens, layer_out=None):
     return logits
 
 
+def latent_attention_core(q_lat, q_rot, c, k_rot, scale, first=0):
+    """q_lat [n, H, C], q_rot [n, H, R] for the positions first .. first + n - 1; c [m, C], k_rot
+    [m, R] every position from 0.  Returns sum_j p_j c_j [n, H, C], p the causal softmax of
+    (q_lat . c_j + q_rot . k_rot_j) * scale."""
+    n, H, C = q_lat.shape
+    out = torch.zeros(n, H, C, dtype=F)
+    for a in range(n):
+        m = first + a + 1
+        for hh in range(H):
+            s = (c[:m] @ q_lat[a, hh] + k_rot[:m] @ q_rot[a, hh]) * scale
+            out[a, hh] = torch.softmax(s, 0) @ c[:m]
+    return out
+
+
+def spread(logits):
+    """Root mean square of the logits around their mean over the vocabulary, averaged over rows."""
+    c = logits - logits.mean(-1, keepdim=True)
+    return float(torch.sqrt((c * c).mean(-1)).mean())
+
+
+def row_errors(got, want):
+    """Per row: rms over the vocabulary of the difference with its mean taken off."""
+    d = got.to(F) - want.to(F)
+    d = d - d.mean(-1, keepdim=True)
+    return torch.sqrt((d * d).mean(-1))
+
+
 # ----------------------------------------------------------------------------- small random models
+def delta_layer(heads, kv_heads, dim, vdim=None, conv=4, mlp=None):
+    return {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim or dim, "conv": conv},
+            "mlp": mlp}
+
+
+def rglru_layer(width, blocks, conv=4, mlp=None):
+    return {"type": "rglru", "mixer": {"width": width, "blocks": blocks, "conv": conv}, "mlp": mlp}
+
+
+def latent_layer(heads, dim, rot_dim, vdim, kv_rank, q_rank, scale=None, base=10000.0, scaling=None, mlp=None):
+    return {"type": "latent_attention",
+            "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+                      "scale": (dim + rot_dim)**-0.5 if scale is None else scale,
+                      "rot": {"base": base, "dims": rot_dim, **({"scaling": scaling} if scaling else {})}},
+            "mlp": mlp}
+
+
+def dense_mlp(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_mlp(experts, top, ff):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def make_config(layers, vocab=97, width=64, eps=1e-5, alpha=1.5, embed_scale=3.0, side_dim=8, softcap=20.0):
+    cfg = {"architecture": "Lamosun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "postln_alpha": alpha,
+           "embedding": {"scale": embed_scale}, "layers": layers}
+    if side_dim:
+        cfg["token_side"] = {"dim": side_dim}
+    if softcap:
+        cfg["logit_softcap"] = softcap
+    return cfg
+
+
 def tensor_shapes(cfg):
     W, V = cfg["width"], cfg["vocab"]
     L = len(cfg["layers"])
@@ -302,3 +380,4 @@ def write_checkpoint(folder, cfg, tensors):
         f.write(hj)
         for b in blobs:
             f.write(b)
+    return folder
