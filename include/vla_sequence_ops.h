@@ -375,6 +375,23 @@ int vla_seq_latent_attention(void* out, int64_t out_token_stride, int64_t out_he
                              int heads, int rank, int rot, int block_size, int num_blocks,
                              float scale, int dtype, void* stream);
 
+/* The same attention on the matrix cores for 16-bit models: 32 query rows that are (token, head)
+ * pairs of one sequence per workgroup, tiles of 32 keys.  rank a multiple of 32 up to 512, rot a
+ * multiple of 16 (vla_seq_latent_attention_tiles_supported); query and cache rows must be 16-byte
+ * aligned.  Rows query_start_loc[b] .. of sequence b sit at positions context_lens[b] ...
+ * vla_seq_set_latent_attention_kernel(1) keeps it off (tests run both), 0 is the default. */
+int vla_seq_latent_attention_tiles_supported(int rank, int rot, int dtype);
+int vla_seq_latent_attention_tiles(void* out, int64_t out_token_stride, int64_t out_head_stride,
+                                   const void* q_lat, int64_t lat_token_stride,
+                                   int64_t lat_head_stride, const void* q_rot,
+                                   int64_t rot_token_stride, int64_t rot_head_stride,
+                                   const void* cache, const int* block_tables, int max_blocks,
+                                   const int* query_start_loc, const int* context_lens,
+                                   int num_seqs, int max_query_len, int heads, int rank, int rot,
+                                   int block_size, int num_blocks, float scale, int dtype,
+                                   void* stream);
+int vla_seq_set_latent_attention_kernel(int mode);
+
 /* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);
  * scan 0 = per shape, 1 = token by token. */
 int vla_seq_set_window_kernel(int mode);

@@ -291,7 +291,7 @@ def test_real_gated_recurrence_short_long_and_cut(channels, blocks, dtype):
 
 # ----------------------------------------------------------------------------- latent attention
 LATENT_SHAPES = [(4, 16, 8, 16, 24), (3, 12, 6, 20, 10), (2, 16, 0, 16, 16), (10, 32, 32, 32, 64), (16, 64, 64, 32, 128),
-                 (40, 32, 32, 16, 96)]
+                 (40, 32, 32, 16, 96), (5, 32, 0, 32, 32), (2, 64, 16, 64, 512), (64, 32, 48, 32, 160)]
 
 
 def latent_layer_of(shape, dtype, scaling=None, seed=0):
@@ -315,6 +315,20 @@ def latent_reference(shape, q, kv, uk, uv, nw, scaling):
     q_lat = torch.einsum("nhd,hdc->nhc", q3[..., :D], uk.view(H, D, C))
     o = R.latent_attention_core(q_lat, q_rot, c, k_rot, 0.3)
     return torch.einsum("nhc,hvc->nhv", o, uv.view(H, V, C)).reshape(n, H * V), c, k_rot
+
+
+@pytest.fixture
+def plain_kernels():
+    """Keeps latent attention off the matrix cores for one test."""
+    from vllm_legacy_amd import _seq_ops as ops
+    ops.set_latent_attention_kernel(1)
+    yield
+    ops.set_latent_attention_kernel(0)
+
+
+@pytest.mark.parametrize("shape", [s for s in LATENT_SHAPES if s[4] % 32 == 0 and s[2] % 16 == 0])
+def test_latent_attention_without_the_matrix_cores(shape, plain_kernels):
+    test_latent_attention_prompt_portions_and_decoding(shape, torch.bfloat16)
 
 
 @pytest.mark.parametrize("shape", LATENT_SHAPES)

@@ -62,7 +62,8 @@ SEQ_EXPORTS = [
     "vla_seq_kv_attention_tiles", "vla_seq_set_kv_attention_kernel", "vla_seq_set_grouped_linear_form",
     "vla_seq_post_norm", "vla_seq_rms_norm_rows", "vla_seq_short_conv", "vla_seq_gated_act_lookup",
     "vla_seq_embed_scaled", "vla_seq_softcap", "vla_seq_delta_rule_scan", "vla_seq_rglru_scan",
-    "vla_seq_latent_rotary_write", "vla_seq_latent_attention",
+    "vla_seq_latent_rotary_write", "vla_seq_latent_attention", "vla_seq_latent_attention_tiles",
+    "vla_seq_latent_attention_tiles_supported", "vla_seq_set_latent_attention_kernel",
 ]
 _seq_lib = None
 
@@ -141,6 +142,10 @@ def seq_lib():
         L.vla_seq_moe_plan.argtypes = [p, i, i, i, p, p, p, i, p]
         L.vla_seq_grouped_linear.argtypes = [p, i64, i, p, i64, p, p, p, i, i, i, i, i, p]
         L.vla_seq_moe_combine.argtypes = [p, p, p, p, p, i64, p, p, i, i, i, i, p]
+        L.vla_seq_latent_attention_tiles_supported.argtypes = [i, i, i]
+        L.vla_seq_latent_attention_tiles.argtypes = [p, i64, i64, p, i64, i64, p, i64, i64, p, p, i, p, p, i, i,
+                                                     i, i, i, i, i, f, i, p]
+        L.vla_seq_set_latent_attention_kernel.argtypes = [i]
         _seq_lib = L
     return _seq_lib
 

@@ -723,3 +723,48 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor
             q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], token_seq.data_ptr(), positions.data_ptr(), T, H, rank, rot, BS, NB, float(scale),
             _dt(q_lat.dtype), _stream(q_lat.device)), "latent_attention")
+
+
+def set_latent_attention_kernel(mode: int) -> None:
+    """0: latent attention picks its kernel per shape; 1: never the matrix-core kernel."""
+    seq_check(_lib.seq_lib().vla_seq_set_latent_attention_kernel(mode), "set_latent_attention_kernel")
+
+
+def latent_attention_tiles_supported(q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor) -> bool:
+    """Whether the matrix-core kernel takes these query tensors and this cache."""
+    rank, rot = q_lat.shape[2], q_rot.shape[2]
+    ok = bool(_lib.seq_lib().vla_seq_latent_attention_tiles_supported(rank, rot, _dt(q_lat.dtype)))
+    for t in (q_lat, q_rot):
+        if t.shape[2] == 0:
+            continue
+        ok = ok and t.data_ptr() % 16 == 0 and all(t.stride(d) % 8 == 0 or t.shape[d] == 1 for d in (0, 1))
+    return ok and cache.data_ptr() % 16 == 0
+
+
+def latent_attention_tiles(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
+                           block_tables: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
+                           max_query_len: int, scale: float) -> None:
+    """The same attention as latent_attention for 16-bit activations on the matrix cores; rows
+    query_start_loc[b] .. of sequence b sit at positions context_lens[b] ..."""
+    _gpu(out, q_lat, q_rot, cache, block_tables, query_start_loc, context_lens)
+    NB, BS, width = cache.shape
+    T, H, rank = q_lat.shape
+    rot = width - rank
+    B = context_lens.numel()
+    assert out.shape == q_lat.shape and q_rot.shape == (T, H, rot) and cache.is_contiguous()
+    assert out.dtype == q_lat.dtype == q_rot.dtype == cache.dtype
+    for t in (out, q_lat, q_rot):
+        assert t.stride(2) == 1 or t.shape[2] == 1
+    for t in (block_tables, query_start_loc, context_lens):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert block_tables.dim() == 2 and block_tables.shape[0] == B and query_start_loc.numel() == B + 1
+
+    def st(t, d):       # a stride that is never used may be anything: make it pass the alignment check
+        return t.stride(d) if t.shape[d] > 1 else 8 * ((t.shape[2] + 7) // 8) * (H if d == 0 else 1)
+
+    with torch.cuda.device(q_lat.device):
+        seq_check(_lib.seq_lib().vla_seq_latent_attention_tiles(
+            out.data_ptr(), st(out, 0), st(out, 1), q_lat.data_ptr(), st(q_lat, 0), st(q_lat, 1),
+            q_rot.data_ptr(), st(q_rot, 0), st(q_rot, 1), cache.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(), B, int(max_query_len), H, rank,
+            rot, BS, NB, float(scale), _dt(q_lat.dtype), _stream(q_lat.device)), "latent_attention_tiles")

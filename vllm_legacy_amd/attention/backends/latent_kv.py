@@ -10,7 +10,9 @@ W_uv,h (sum_j p_j c_j).  Rotation: interleaved pairs (2i, 2i + 1) of the first `
 of the rotated parts turn by position * f_i, sine and cosine times `magnitude` (a frequency table
 and a magnitude as YaRN scaling gives them, or plain ones).  `scale` multiplies the scores as it
 is.  Prompts, portions of prompts and decode steps are one case: the step's rows are written to
-the cache, then every query row reads from there (csrc/seq_latent_attention.hip).
+the cache, then every query row reads from there (csrc/seq_latent_attention.hip: a matrix-core
+kernel for 16-bit models whose rank is a multiple of 32 and whose rotated part is a multiple of 16,
+and an fp32 kernel for any dtype and size).
 """
 import math
 from typing import Dict, Optional, Tuple
@@ -88,7 +90,13 @@ class LatentKVAttention(nn.Module):
         q3 = q.view(T, H, D + Rr)
         q_lat = torch.bmm(q3[:, :, :D].transpose(0, 1), self.w_uk.data)             # [H, T, C]
         o_lat = torch.empty((H, T, C), dtype=q.dtype, device=q.device)
-        ops.latent_attention(o_lat.transpose(0, 1), q_lat.transpose(0, 1), q3[:, :, D:], cache, batch.block_tables,
-                             batch.token_seq, batch.positions, self.scale)
+        q_lat, q_rot, o_rows = q_lat.transpose(0, 1), q3[:, :, D:], o_lat.transpose(0, 1)
+        if ops.latent_attention_tiles_supported(q_lat, q_rot, cache):
+            # 16-bit models whose sizes fit: (token, head) rows in tiles of 32 on the matrix cores
+            ops.latent_attention_tiles(o_rows, q_lat, q_rot, cache, batch.block_tables, batch.query_start_loc,
+                                       batch.context_lens, batch.max_query_len, self.scale)
+        else:
+            ops.latent_attention(o_rows, q_lat, q_rot, cache, batch.block_tables, batch.token_seq, batch.positions,
+                                 self.scale)
         o = torch.bmm(o_lat, self.w_uv_t.data)                                      # [H, T, V]
         return o.transpose(0, 1).reshape(T, H * V)

@@ -14,6 +14,8 @@
 // latent_attention_kernel: one wave per (token, head), any dtype, rank up to 1024.  A tile is 64
 // keys: lane j scores key j against the query held in LDS, the wave reduces max / sum (online
 // softmax across tiles), then lane d accumulates sum_j p_j c_j[d] with coalesced reads.
+#include <atomic>
+
 #include "seq_common.h"
 
 namespace vla {
@@ -158,6 +160,294 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// latent_attention_tile_kernel<S, VBW>: 16-bit models on 32x32x16 MFMAs, prompts, portions and
+// decode steps alike.  Every head reads the same cache rows, so a workgroup takes 32 query rows
+// that are (token, head) pairs of one sequence -- up to 32 heads of one token, or all heads of
+// 32 / heads consecutive tokens -- and walks the keys from the first to the last row's position in
+// tiles of 32, staged through LDS once for its four waves (loaded one tile ahead; the rows' places
+// in the paged cache are looked up two tiles ahead).  Both products run in transposed form, lane =
+// (hf, c) = (lane >> 5, lane & 31):
+//   S^T = K q^T   A = K    lane: key c, dims 16 ks + 8 hf .. + 7       (LDS, 16 bytes)
+//                 B = q^T  lane: query row c, the same dims           (LDS, 16 bytes)
+//                 C        lane: query row c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
+//   O^T = C^T P^T B = P^T  lane: query row c, registers 8 s .. 8 s + 7 of C
+//                 A = C^T  lane: latent dim 32 n + c of the same eight keys (two transposing reads
+//                          of the row-major tile: the latent is key and value at once)
+// The four waves split the first product's k-steps (rank + rot dims) and add their partial scores
+// through LDS, so each holds the whole 32 x 32 score block and the same running max and sum; they
+// split the second product's blocks of 32 latent dims (wave w owns blocks w, w + 4, ...).  Scores,
+// max / sum (base 2) and accumulators are fp32; a weight enters the second product rounded to the
+// model dtype.
+template <class S>
+struct LatentMfma;
+template <>
+struct LatentMfma<BF16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
+};
+template <>
+struct LatentMfma<F16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+};
+
+constexpr int kTileKeys = 32;
+constexpr int kTileRows = 32;
+typedef short lat_s16x4 __attribute__((ext_vector_type(4)));
+typedef lat_s16x4 __attribute__((address_space(3))) * lat_lds_s16x4;
+
+template <class S, int VBW>
+__global__ __launch_bounds__(256) void latent_attention_tile_kernel(
+    typename S::T* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride,
+    LatentQuery<S> q, const typename S::T* __restrict__ cache, const int* __restrict__ block_tables,
+    int max_blocks, const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
+    int heads, int rank, int rot, int block_size, int num_blocks, float scale, int hb, int tb) {
+  using T = typename S::T;
+  using M = LatentMfma<S>;
+  constexpr int WP = 2 * VBW + 2;                      // 16-byte pieces of a tile a thread stages
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int width = rank + rot, row_elems = width + 8;   // rows stay 16-byte aligned
+  const int row_pieces = width / 8, tile_pieces = kTileKeys * row_pieces;
+  T* q_lds = reinterpret_cast<T*>(smem);                                     // [32][row_elems]
+  T* k_lds2 = q_lds + kTileRows * row_elems;                                 // [2][32][row_elems]
+  float* s_lds = reinterpret_cast<float*>(k_lds2 + 2 * kTileKeys * row_elems);   // [4][4][64][4]
+  long long* rows_lds = reinterpret_cast<long long*>(s_lds + 4 * 16 * 64);   // [2][32]
+  const int b = blockIdx.z;
+  // the last tiles of a run have the most keys to walk: they are dispatched first
+  const int tile_x = gridDim.x - 1 - blockIdx.x;
+  const int run = query_start_loc[b + 1] - query_start_loc[b];
+  const int tq0 = tile_x * tb;
+  if (tq0 >= run) return;
+  const int ntok = min(tb, run - tq0);
+  const int h0 = blockIdx.y * hb, nh = min(hb, heads - h0);
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int hf = lane >> 5, c = lane & 31;
+  const int t_first = query_start_loc[b] + tq0;
+  const int p_first = context_lens[b] + tq0, p_last = p_first + ntok - 1;
+  const int my_tok = c / hb, my_head = c - my_tok * hb;
+  const bool my_row = my_tok < ntok && my_head < nh;
+  const int pq = p_first + my_tok;
+  const int* table = block_tables + (int64_t)b * max_blocks;
+  const float scale2 = scale * 1.4426950408889634f;    // scores in base 2
+
+  for (int i = tid; i < kTileRows * row_pieces; i += 256) {
+    const int r = i / row_pieces, v = i - r * row_pieces;
+    const int tok = r / hb, hd = r - tok * hb;
+    u32x4 val = {0u, 0u, 0u, 0u};
+    if (tok < ntok && hd < nh) {
+      const int64_t t = t_first + tok, h = h0 + hd;
+      val = 8 * v < rank
+                ? *reinterpret_cast<const u32x4*>(q.lat + t * q.lat_token_stride + h * q.lat_head_stride + 8 * v)
+                : *reinterpret_cast<const u32x4*>(q.rot + t * q.rot_token_stride + h * q.rot_head_stride + 8 * v - rank);
+    }
+    *reinterpret_cast<u32x4*>(q_lds + r * row_elems + 8 * v) = val;
+  }
+  f32x16 o[VBW];
+#pragma unroll
+  for (int n = 0; n < VBW; ++n)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[n][i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  // threads 0 .. 31 look the rows of a tile up: the block id is read one step before it is used
+  auto load_block = [&](int j0) {
+    const int j = j0 + tid;
+    int blk = -1;
+    if (j <= p_last) {
+      blk = table[j / block_size];
+      blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
+    }
+    return blk;
+  };
+  auto store_row = [&](int j0, int blk, int buf) {
+    const int j = j0 + tid;
+    rows_lds[buf * kTileKeys + tid] = blk < 0 ? -1 : (long long)blk * block_size + j % block_size;
+  };
+  u32x4 stage[WP];
+  auto fetch = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WP; ++u) {
+      const int i = tid + 256 * u;
+      u32x4 got = {0u, 0u, 0u, 0u};
+      if (i < tile_pieces) {
+        const int r = i / row_pieces, v = i - r * row_pieces;
+        const long long row = rows_lds[buf * kTileKeys + r];
+        if (row >= 0) got = *reinterpret_cast<const u32x4*>(cache + row * width + 8 * v);
+      }
+      stage[u] = got;
+    }
+  };
+  auto land = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WP; ++u) {
+      const int i = tid + 256 * u;
+      if (i < tile_pieces) {
+        const int r = i / row_pieces, v = i - r * row_pieces;
+        *reinterpret_cast<u32x4*>(k_lds2 + (buf * kTileKeys + r) * row_elems + 8 * v) = stage[u];
+      }
+    }
+  };
+  // One barrier pair per tile.  At the top of step `it`: tile `it` is in LDS buffer it & 1, tile
+  // it + 1 in the staging registers, the rows of tile it + 2 in rows_lds[it & 1], and threads
+  // 0 .. 31 hold the block ids of tile it + 3.
+  int blk_next = -1;
+  if (tid < kTileKeys) {
+    store_row(0, load_block(0), 0);
+    store_row(kTileKeys, load_block(kTileKeys), 1);
+  }
+  __syncthreads();
+  fetch(0);
+  land(0);
+  fetch(1);
+  __syncthreads();
+  if (tid < kTileKeys) {
+    store_row(2 * kTileKeys, load_block(2 * kTileKeys), 0);
+    blk_next = load_block(3 * kTileKeys);
+  }
+  __syncthreads();
+  const int ksteps = width / 16, vb = rank / 32;
+  int it = 0;
+  for (int j0 = 0; j0 <= p_last; j0 += kTileKeys, ++it) {
+    const T* k_lds = k_lds2 + (it & 1) * kTileKeys * row_elems;
+    f32x16 st;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st[i] = 0.f;
+    for (int ks = w; ks < ksteps; ks += 4) {
+      const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + c * row_elems + 16 * ks + 8 * hf);
+      const u32x4 bq = *reinterpret_cast<const u32x4*>(q_lds + c * row_elems + 16 * ks + 8 * hf);
+      st = M::run(a, bq, st);
+    }
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const f32x4 part = {st[4 * i4], st[4 * i4 + 1], st[4 * i4 + 2], st[4 * i4 + 3]};
+      *reinterpret_cast<f32x4*>(s_lds + ((w * 4 + i4) * 64 + lane) * 4) = part;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ow = 1; ow < 4; ++ow) {
+      const int w2 = (w + ow) & 3;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const f32x4 part = *reinterpret_cast<const f32x4*>(s_lds + ((w2 * 4 + i4) * 64 + lane) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st[4 * i4 + e] += part[e];
+      }
+    }
+    // (the sum above runs in a different order in each wave; every wave keeps its own max and sum, and
+    // they only need to agree with its own weights)
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int j = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      const float v = my_row && j <= pq ? st[i] * scale2 : -INFINITY;
+      st[i] = v;
+      mt = fmaxf(mt, v);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const bool none = m_new == -INFINITY;
+    const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float pv = none ? 0.f : __builtin_amdgcn_exp2f(st[i] - m_new);
+      st[i] = pv;
+      psum += pv;
+    }
+    l = l * corr + psum;            // this lane's keys; the partner's half is added at the end
+    m = m_new;
+    if (__any(corr != 1.f)) {
+#pragma unroll
+      for (int n = 0; n < VBW; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[n][i] *= corr;
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      u32x4 pb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pb[e] = M::pack2(st[8 * s2 + 2 * e], st[8 * s2 + 2 * e + 1]);
+      // transposing read of the row-major tile: a group of 16 lanes reads 4 keys x 16 dims, 8
+      // bytes per lane, and every lane receives the four keys of one dim of the group
+      const int i16 = c & 15;
+      const T* src = k_lds + (16 * s2 + 4 * hf + (i16 >> 2)) * row_elems + 16 * (c >> 4) + 4 * (i16 & 3);
+#pragma unroll
+      for (int n = 0; n < VBW; ++n) {
+        const int blk = w + 4 * n;
+        if (blk < vb) {
+          const lat_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lat_lds_s16x4)(src + 32 * blk));
+          const lat_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lat_lds_s16x4)(src + 32 * blk + 8 * row_elems));
+          const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+          const u32x4 a = {lo2[0], lo2[1], hi2[0], hi2[1]};
+          o[n] = M::run(a, pb, o[n]);
+        }
+      }
+    }
+    if (j0 + kTileKeys <= p_last) land((it + 1) & 1);            // tile it + 1, fetched a step ago
+    if (j0 + 2 * kTileKeys <= p_last) fetch(it & 1);             // tile it + 2 on its way
+    if (tid < kTileKeys && j0 + 3 * kTileKeys <= p_last) {
+      store_row(j0 + 3 * kTileKeys, blk_next, (it + 1) & 1);
+      blk_next = load_block(j0 + 4 * kTileKeys);
+    }
+    __syncthreads();
+  }
+  l += __shfl_xor(l, 32, 64);
+  if (!my_row) return;
+  const float inv = 1.f / l;
+  T* orow = out + (int64_t)(t_first + my_tok) * out_token_stride + (int64_t)(h0 + my_head) * out_head_stride;
+#pragma unroll
+  for (int n = 0; n < VBW; ++n) {
+    const int blk = w + 4 * n;
+    if (blk < vb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        orow[32 * blk + (i & 3) + 8 * (i >> 2) + 4 * hf] = S::from_f32(o[n][i] * inv);
+    }
+  }
+}
+
+std::atomic<int> g_latent_kernel{0};
+
+bool latent_tile_sizes(int rank, int rot) {
+  if (rank % 32 != 0 || rank < 32 || rank > 512 || rot % 16 != 0) return false;
+  const int vbw = (rank / 32 + 3) / 4;
+  return (rank + rot) * kTileKeys / 8 <= 256 * (2 * vbw + 2);
+}
+
+template <class S, int VBW>
+int launch_latent_tiles(dim3 grid, size_t lds, hipStream_t stream, typename S::T* out,
+                        int64_t out_token_stride, int64_t out_head_stride, const LatentQuery<S>& q,
+                        const typename S::T* cache, const int* block_tables, int max_blocks,
+                        const int* qsl, const int* ctx, int heads, int rank, int rot, int block_size,
+                        int num_blocks, float scale, int hb, int tb) {
+  static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
+  if (lds > allowed.load(std::memory_order_relaxed)) {
+    VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&latent_attention_tile_kernel<S, VBW>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    allowed.store(lds, std::memory_order_relaxed);
+  }
+  latent_attention_tile_kernel<S, VBW><<<grid, 256, lds, stream>>>(
+      out, out_token_stride, out_head_stride, q, cache, block_tables, max_blocks, qsl, ctx, heads,
+      rank, rot, block_size, num_blocks, scale, hb, tb);
+  VLA_SEQ_HIP_CHECK(hipGetLastError());
+  return VLA_OK;
+}
+
 }  // namespace
 }  // namespace seq
 }  // namespace vla
@@ -219,4 +509,63 @@ extern "C" int vla_seq_latent_attention(void* out, int64_t out_token_stride, int
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
+}
+
+// 0: pick per shape; 1: never the matrix-core kernel (tests run both)
+extern "C" int vla_seq_set_latent_attention_kernel(int mode) {
+  if (mode < 0 || mode > 1) return VLA_ERR_ARG;
+  g_latent_kernel.store(mode, std::memory_order_relaxed);
+  return VLA_OK;
+}
+
+extern "C" int vla_seq_latent_attention_tiles_supported(int rank, int rot, int dtype) {
+  return (dtype == VLA_F16 || dtype == VLA_BF16) && latent_tile_sizes(rank, rot) &&
+         g_latent_kernel.load(std::memory_order_relaxed) == 0;
+}
+
+extern "C" int vla_seq_latent_attention_tiles(
+    void* out, int64_t out_token_stride, int64_t out_head_stride, const void* q_lat,
+    int64_t lat_token_stride, int64_t lat_head_stride, const void* q_rot, int64_t rot_token_stride,
+    int64_t rot_head_stride, const void* cache, const int* block_tables, int max_blocks,
+    const int* query_start_loc, const int* context_lens, int num_seqs, int max_query_len, int heads,
+    int rank, int rot, int block_size, int num_blocks, float scale, int dtype, void* stream) {
+  if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
+  if (!out || !q_lat || (rot > 0 && !q_rot) || !cache || !block_tables || !query_start_loc ||
+      !context_lens || num_seqs < 0 || num_seqs > 65535 || max_query_len < 0 || heads <= 0 ||
+      rot < 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0)
+    return VLA_ERR_ARG;
+  if ((dtype != VLA_F16 && dtype != VLA_BF16) || !latent_tile_sizes(rank, rot)) return VLA_ERR_HEAD_SIZE;
+  // 16-byte fragment loads: query rows and cache rows must allow them
+  if (((uintptr_t)q_lat % 16) || (lat_token_stride % 8) || (lat_head_stride % 8) || ((uintptr_t)cache % 16) ||
+      (rot > 0 && (((uintptr_t)q_rot % 16) || (rot_token_stride % 8) || (rot_head_stride % 8))))
+    return VLA_ERR_ARG;
+  const int hb = heads < kTileRows ? heads : kTileRows;     // heads of a workgroup's rows
+  const int tb = kTileRows / hb;                            // tokens of a workgroup's rows
+  const dim3 grid((max_query_len + tb - 1) / tb, (heads + hb - 1) / hb, num_seqs);
+  const int row_elems = rank + rot + 8;
+  const size_t lds = (size_t)3 * kTileRows * row_elems * 2 + 4 * 16 * 64 * sizeof(float) +
+                     2 * kTileKeys * sizeof(long long);
+  if (lds > 160 * 1024) return VLA_ERR_HEAD_SIZE;
+  const int vbw = (rank / 32 + 3) / 4;
+  auto go = [&](auto s) {
+    using S = decltype(s);
+    using T = typename S::T;
+    const LatentQuery<S> q{(const T*)q_lat, lat_token_stride, lat_head_stride, (const T*)q_rot,
+                           rot_token_stride, rot_head_stride};
+#define VLA_LATENT_CASE(N)                                                                          \
+  case N:                                                                                           \
+    return launch_latent_tiles<S, N>(grid, lds, (hipStream_t)stream, (T*)out, out_token_stride,     \
+                                     out_head_stride, q, (const T*)cache, block_tables, max_blocks, \
+                                     query_start_loc, context_lens, heads, rank, rot, block_size,   \
+                                     num_blocks, scale, hb, tb);
+    switch (vbw) {
+      VLA_LATENT_CASE(1)
+      VLA_LATENT_CASE(2)
+      VLA_LATENT_CASE(3)
+      VLA_LATENT_CASE(4)
+      default: return (int)VLA_ERR_HEAD_SIZE;
+    }
+#undef VLA_LATENT_CASE
+  };
+  return dtype == VLA_BF16 ? go(BF16{}) : go(F16{});
 }
