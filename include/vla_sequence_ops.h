@@ -321,16 +321,22 @@ int vla_seq_softcap(float* z, int64_t n, float cap, void* stream);
  * softplus(dt row + dt_bias)); out = out_dtype(o / sqrt(mean_v(o^2) + eps) * norm_weight *
  * silu(gate)).  q, k [T, kv_heads * dim], v, gate, out [T, heads * vdim], beta, dt [T, heads]:
  * rows with their own strides, inputs fp32 (in_dtype VLA_F32).  A sequence with context 0 starts
- * from zero.  vdim * (dim / 64 rounded up to a power of two) <= 1024. */
+ * from zero.  scratch: fp32, vla_seq_delta_rule_scratch_floats values (the heads' outputs between
+ * the walk and their norm).  max_query_len: the longest run of the step (0: unknown).  dim up to
+ * 1024. */
+int64_t vla_seq_delta_rule_scratch_floats(int num_tokens, int heads, int vdim);
+/* Kernel choice for tests: 0 = per step (runs of at most four rows skip the LDS staging), 1 = always
+ * without staging, 2 = never. */
+int vla_seq_set_delta_kernel(int mode);
 int vla_seq_delta_rule_scan(void* out, int64_t out_stride, int out_dtype, const void* q,
                             int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                             int64_t v_stride, const void* gate, int64_t gate_stride,
                             const void* beta, int64_t beta_stride, const void* dt, int64_t dt_stride,
                             int in_dtype, const float* a_log, const float* dt_bias,
                             const float* norm_weight, float* state, const int* query_start_loc,
-                            const int* context_lens, const int* state_slots, int num_seqs,
-                            int num_slots, int heads, int kv_heads, int dim, int vdim, float eps,
-                            void* stream);
+                            const int* context_lens, const int* state_slots, int num_tokens,
+                            int num_seqs, int max_query_len, int num_slots, int heads, int kv_heads,
+                            int dim, int vdim, float eps, float* scratch, void* stream);
 
 /* ---- real-gated linear recurrent unit ------------------------------------------------------------- */
 

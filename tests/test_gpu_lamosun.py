@@ -233,11 +233,18 @@ def run_delta(H, G, D, V, rows, cuts, seed=0, craft=None):
 
 
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (3, 1, 24, 40), (2, 2, 128, 128), (1, 1, 200, 72), (5, 5, 8, 12)])
-def test_delta_rule_whole_cut_and_token_by_token(shape):
+@pytest.mark.parametrize("kernel", [0, 1, 2])
+def test_delta_rule_whole_cut_and_token_by_token(shape, kernel):
+    """kernel 0: as a step picks it; 1: every run on the kernel for short runs; 2: every run staged."""
+    from vllm_legacy_amd import _seq_ops as ops
     rows = 45
-    for cuts in ([rows], [2, 17, 3, 23], [1] * rows):
-        got, want = run_delta(*shape, rows, cuts)
-        close(got, want, 3e-5, (shape, cuts[:3]))
+    ops.set_delta_kernel(kernel)
+    try:
+        for cuts in ([rows], [2, 17, 3, 23], [1] * rows):
+            got, want = run_delta(*shape, rows, cuts)
+            close(got, want, 3e-5, (shape, cuts[:3]))
+    finally:
+        ops.set_delta_kernel(0)
 
 
 def test_delta_rule_reads_a_write_from_hundreds_of_tokens_back():

@@ -61,7 +61,7 @@ SEQ_EXPORTS = [
     "vla_seq_grouped_linear", "vla_seq_moe_combine", "vla_seq_kv_attention_tiles_supported",
     "vla_seq_kv_attention_tiles", "vla_seq_set_kv_attention_kernel", "vla_seq_set_grouped_linear_form",
     "vla_seq_post_norm", "vla_seq_rms_norm_rows", "vla_seq_short_conv", "vla_seq_gated_act_lookup",
-    "vla_seq_embed_scaled", "vla_seq_softcap", "vla_seq_delta_rule_scan", "vla_seq_rglru_scan",
+    "vla_seq_embed_scaled", "vla_seq_softcap", "vla_seq_delta_rule_scan", "vla_seq_delta_rule_scratch_floats", "vla_seq_set_delta_kernel", "vla_seq_rglru_scan",
     "vla_seq_latent_rotary_write", "vla_seq_latent_attention", "vla_seq_latent_attention_tiles",
     "vla_seq_latent_attention_tiles_supported", "vla_seq_set_latent_attention_kernel",
 ]
@@ -131,7 +131,10 @@ def seq_lib():
         L.vla_seq_embed_scaled.argtypes = [p, p, p, f, i, i, i, i, p]
         L.vla_seq_softcap.argtypes = [p, i64, f, p]
         L.vla_seq_delta_rule_scan.argtypes = [p, i64, i, p, i64, p, i64, p, i64, p, i64, p, i64, p, i64, i,
-                                              p, p, p, p, p, p, p, i, i, i, i, i, i, f, p]
+                                              p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, p, p]
+        L.vla_seq_delta_rule_scratch_floats.argtypes = [i, i, i]
+        L.vla_seq_delta_rule_scratch_floats.restype = i64
+        L.vla_seq_set_delta_kernel.argtypes = [i]
         L.vla_seq_rglru_scan.argtypes = [p, i64, i, p, i64, p, i64, i, i64, p, i64, p, i64, p, p, p, p, p, i, i,
                                          i, i, p, i64, p]
         L.vla_seq_latent_rotary_write.argtypes = [p, i64, i, i, p, i64, p, f, p, p, p, p, f, i, i, i, i, i,

@@ -621,7 +621,8 @@ def softcap(z: torch.Tensor, cap: float) -> None:
 def delta_rule_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
                     beta: torch.Tensor, dt: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                     norm_weight: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor,
-                    context_lens: torch.Tensor, state_slots: torch.Tensor, kv_heads: int, eps: float) -> None:
+                    context_lens: torch.Tensor, state_slots: torch.Tensor, kv_heads: int, eps: float,
+                    max_query_len: int = 0) -> None:
     """out [T, H*V]; q, k fp32 [T, G*D]; v, gate fp32 [T, H*V]; beta, dt fp32 [T, H] (views with free
     row strides); a_log, dt_bias fp32 [H]; norm_weight fp32 [V]; state fp32 [slots, H, V, D]."""
     _gpu(out, q, k, v, gate, beta, dt, a_log, dt_bias, norm_weight, state, query_start_loc, context_lens, state_slots)
@@ -636,14 +637,22 @@ def delta_rule_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torc
     for t in (query_start_loc, context_lens, state_slots):
         assert t.dtype == torch.int32 and t.is_contiguous()
     assert query_start_loc.numel() == B + 1 and state_slots.numel() == B
+    T = q.shape[0]
+    scratch = torch.empty(_lib.seq_lib().vla_seq_delta_rule_scratch_floats(T, H, V), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         seq_check(_lib.seq_lib().vla_seq_delta_rule_scan(
             out.data_ptr(), _rows(out, H * V), _dt(out.dtype), q.data_ptr(), _rows(q, kv_heads * D), k.data_ptr(),
             _rows(k, kv_heads * D), v.data_ptr(), _rows(v, H * V), gate.data_ptr(), _rows(gate, H * V),
             beta.data_ptr(), _rows(beta, H), dt.data_ptr(), _rows(dt, H), _lib.F32, a_log.data_ptr(),
             dt_bias.data_ptr(), norm_weight.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
-            context_lens.data_ptr(), state_slots.data_ptr(), B, slots, H, int(kv_heads), D, V, float(eps),
-            _stream(q.device)), "delta_rule_scan")
+            context_lens.data_ptr(), state_slots.data_ptr(), T, B, int(max_query_len), slots, H, int(kv_heads), D, V,
+            float(eps),
+            scratch.data_ptr(), _stream(q.device)), "delta_rule_scan")
+
+
+def set_delta_kernel(mode: int) -> None:
+    """0: delta_rule_scan picks its kernel per step; 1: always the one without staging; 2: never."""
+    seq_check(_lib.seq_lib().vla_seq_set_delta_kernel(mode), "set_delta_kernel")
 
 
 def rglru_scan(out: torch.Tensor, gates: torch.Tensor, u: torch.Tensor, y: torch.Tensor,

@@ -182,7 +182,7 @@ class GatedDeltaRule(nn.Module):
         """q, k [T, G*D]; v, gate, out [T, H*V]; beta, dt [T, H]: views with free row strides."""
         ops.delta_rule_scan(out, q, k, v, gate, beta, dt, self.a_log.data, self.dt_bias.data, self.norm_weight.data,
                             state, batch.query_start_loc, batch.context_lens, batch.state_slots, self.kv_heads,
-                            self.eps)
+                            self.eps, batch.max_query_len)
         return out
 
 
