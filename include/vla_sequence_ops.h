@@ -385,8 +385,12 @@ int vla_seq_latent_attention(void* out, int64_t out_token_stride, int64_t out_he
  * pairs of one sequence per workgroup, tiles of 32 keys.  rank a multiple of 32 up to 512, rot a
  * multiple of 16 (vla_seq_latent_attention_tiles_supported); query and cache rows must be 16-byte
  * aligned.  Rows query_start_loc[b] .. of sequence b sit at positions context_lens[b] ...
+ * key_splits > 1 shares the keys of every row tile out to that many workgroups and merges their
+ * sums in a second launch (few rows over long contexts); scratch then holds
+ * vla_seq_latent_attention_scratch_floats fp32 values and num_tokens is the step's row count.
  * vla_seq_set_latent_attention_kernel(1) keeps it off (tests run both), 0 is the default. */
 int vla_seq_latent_attention_tiles_supported(int rank, int rot, int dtype);
+int64_t vla_seq_latent_attention_scratch_floats(int key_splits, int num_tokens, int heads, int rank);
 int vla_seq_latent_attention_tiles(void* out, int64_t out_token_stride, int64_t out_head_stride,
                                    const void* q_lat, int64_t lat_token_stride,
                                    int64_t lat_head_stride, const void* q_rot,
@@ -394,8 +398,8 @@ int vla_seq_latent_attention_tiles(void* out, int64_t out_token_stride, int64_t 
                                    const void* cache, const int* block_tables, int max_blocks,
                                    const int* query_start_loc, const int* context_lens,
                                    int num_seqs, int max_query_len, int heads, int rank, int rot,
-                                   int block_size, int num_blocks, float scale, int dtype,
-                                   void* stream);
+                                   int block_size, int num_blocks, float scale, int key_splits,
+                                   float* scratch, int num_tokens, int dtype, void* stream);
 int vla_seq_set_latent_attention_kernel(int mode);
 
 /* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);

@@ -188,7 +188,7 @@ def run(args):
             o_lat = torch.empty(H, T, Cr, device=dev, dtype=dt).transpose(0, 1)
             sec = timed(lambda: sops.latent_attention_tiles(o_lat, q_lat, q_rot, latent, batch.block_tables,
                                                             batch.query_start_loc, batch.context_lens,
-                                                            batch.max_query_len, attn.scale), it)
+                                                            batch.max_query_len, attn.scale, attn.key_splits(batch)), it)
             if tag == "prefill":
                 record(kern, "lamosun.latent_attention.prefill", sec, flops=2.0 * (T * (T + 1) / 2) * H * (Wl + Cr),
                        nbytes=2.0 * T * (H * (Wl + Cr) + Wl),

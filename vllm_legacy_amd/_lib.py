@@ -63,7 +63,7 @@ SEQ_EXPORTS = [
     "vla_seq_post_norm", "vla_seq_rms_norm_rows", "vla_seq_short_conv", "vla_seq_gated_act_lookup",
     "vla_seq_embed_scaled", "vla_seq_softcap", "vla_seq_delta_rule_scan", "vla_seq_delta_rule_scratch_floats", "vla_seq_set_delta_kernel", "vla_seq_rglru_scan",
     "vla_seq_latent_rotary_write", "vla_seq_latent_attention", "vla_seq_latent_attention_tiles",
-    "vla_seq_latent_attention_tiles_supported", "vla_seq_set_latent_attention_kernel",
+    "vla_seq_latent_attention_tiles_supported", "vla_seq_latent_attention_scratch_floats", "vla_seq_set_latent_attention_kernel",
 ]
 _seq_lib = None
 
@@ -147,7 +147,9 @@ def seq_lib():
         L.vla_seq_moe_combine.argtypes = [p, p, p, p, p, i64, p, p, i, i, i, i, p]
         L.vla_seq_latent_attention_tiles_supported.argtypes = [i, i, i]
         L.vla_seq_latent_attention_tiles.argtypes = [p, i64, i64, p, i64, i64, p, i64, i64, p, p, i, p, p, i, i,
-                                                     i, i, i, i, i, f, i, p]
+                                                     i, i, i, i, i, f, i, p, i, i, p]
+        L.vla_seq_latent_attention_scratch_floats.argtypes = [i, i, i, i]
+        L.vla_seq_latent_attention_scratch_floats.restype = i64
         L.vla_seq_set_latent_attention_kernel.argtypes = [i]
         _seq_lib = L
     return _seq_lib

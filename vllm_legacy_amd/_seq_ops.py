@@ -752,9 +752,10 @@ def latent_attention_tiles_supported(q_lat: torch.Tensor, q_rot: torch.Tensor, c
 
 def latent_attention_tiles(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
                            block_tables: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
-                           max_query_len: int, scale: float) -> None:
+                           max_query_len: int, scale: float, key_splits: int = 1) -> None:
     """The same attention as latent_attention for 16-bit activations on the matrix cores; rows
-    query_start_loc[b] .. of sequence b sit at positions context_lens[b] ..."""
+    query_start_loc[b] .. of sequence b sit at positions context_lens[b] ...  key_splits > 1: the
+    keys of every row tile are shared out to that many workgroups and merged."""
     _gpu(out, q_lat, q_rot, cache, block_tables, query_start_loc, context_lens)
     NB, BS, width = cache.shape
     T, H, rank = q_lat.shape
@@ -771,9 +772,13 @@ def latent_attention_tiles(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.
     def st(t, d):       # a stride that is never used may be anything: make it pass the alignment check
         return t.stride(d) if t.shape[d] > 1 else 8 * ((t.shape[2] + 7) // 8) * (H if d == 0 else 1)
 
+    L = _lib.seq_lib()
+    need = L.vla_seq_latent_attention_scratch_floats(int(key_splits), T, H, rank)
+    scratch = torch.empty(need, dtype=torch.float32, device=q_lat.device) if need else None
     with torch.cuda.device(q_lat.device):
-        seq_check(_lib.seq_lib().vla_seq_latent_attention_tiles(
+        seq_check(L.vla_seq_latent_attention_tiles(
             out.data_ptr(), st(out, 0), st(out, 1), q_lat.data_ptr(), st(q_lat, 0), st(q_lat, 1),
             q_rot.data_ptr(), st(q_rot, 0), st(q_rot, 1), cache.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(), B, int(max_query_len), H, rank,
-            rot, BS, NB, float(scale), _dt(q_lat.dtype), _stream(q_lat.device)), "latent_attention_tiles")
+            rot, BS, NB, float(scale), int(key_splits), _p(scratch), T, _dt(q_lat.dtype), _stream(q_lat.device)),
+            "latent_attention_tiles")

@@ -75,6 +75,20 @@ class LatentKVAttention(nn.Module):
         self.w_uv_t.data = uv.to(self.dtype).view(H, V, C).transpose(1, 2).to(dev).contiguous()
         self.latent_norm.data = latent_norm.float().to(dev).contiguous()
 
+    # workgroups a launch should have before the keys of a row tile stay with one workgroup
+    SPLIT_BELOW_WORKGROUPS = 1024
+    KEYS_PER_SPLIT = 256
+
+    def key_splits(self, batch: SequenceBatch) -> int:
+        """Steps of few rows over long contexts (decode steps) share every row tile's keys out to
+        several workgroups: enough of them to fill the part, none with fewer than KEYS_PER_SPLIT
+        keys."""
+        heads_per = min(self.num_heads, 32)
+        tiles = -(-batch.max_query_len // (32 // heads_per)) * -(-self.num_heads // heads_per) * batch.num_seqs
+        if tiles >= self.SPLIT_BELOW_WORKGROUPS:
+            return 1
+        return max(1, min(-(-self.SPLIT_BELOW_WORKGROUPS // tiles), batch.max_seq_len // self.KEYS_PER_SPLIT, 32))
+
     @staticmethod
     def get_cache_shape(num_blocks: int, block_size: int, rank: int, rot_dim: int) -> Tuple[int, ...]:
         return (num_blocks, block_size, rank + rot_dim)
@@ -94,7 +108,8 @@ class LatentKVAttention(nn.Module):
         if ops.latent_attention_tiles_supported(q_lat, q_rot, cache):
             # 16-bit models whose sizes fit: (token, head) rows in tiles of 32 on the matrix cores
             ops.latent_attention_tiles(o_rows, q_lat, q_rot, cache, batch.block_tables, batch.query_start_loc,
-                                       batch.context_lens, batch.max_query_len, self.scale)
+                                       batch.context_lens, batch.max_query_len, self.scale,
+                                       self.key_splits(batch))
         else:
             ops.latent_attention(o_rows, q_lat, q_rot, cache, batch.block_tables, batch.token_seq, batch.positions,
                                  self.scale)

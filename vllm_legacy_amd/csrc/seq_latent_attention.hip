@@ -166,11 +166,12 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
 // decode steps alike.  Every head reads the same cache rows, so a workgroup takes 32 query rows
 // that are (token, head) pairs of one sequence -- up to 32 heads of one token, or all heads of
 // 32 / heads consecutive tokens -- and walks the keys from the first to the last row's position in
-// tiles of 32, staged through LDS once for its four waves (loaded one tile ahead; the rows' places
-// in the paged cache are looked up two tiles ahead).  Both products run in transposed form, lane =
+// tiles of 32, staged through LDS once for its four waves (loaded one tile ahead into registers; the
+// rows' places in the paged cache are looked up two tiles ahead).  One tile and the partial scores
+// are all the LDS a workgroup holds, so two workgroups share a CU.  Both products run in transposed form, lane =
 // (hf, c) = (lane >> 5, lane & 31):
 //   S^T = K q^T   A = K    lane: key c, dims 16 ks + 8 hf .. + 7       (LDS, 16 bytes)
-//                 B = q^T  lane: query row c, the same dims           (LDS, 16 bytes)
+//                 B = q^T  lane: query row c, the same dims           (registers, loaded once)
 //                 C        lane: query row c, keys (i & 3) + 8 (i >> 2) + 4 hf, i = 0 .. 15
 //   O^T = C^T P^T B = P^T  lane: query row c, registers 8 s .. 8 s + 7 of C
 //                 A = C^T  lane: latent dim 32 n + c of the same eight keys (two transposing reads
@@ -179,7 +180,8 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
 // through LDS, so each holds the whole 32 x 32 score block and the same running max and sum; they
 // split the second product's blocks of 32 latent dims (wave w owns blocks w, w + 4, ...).  Scores,
 // max / sum (base 2) and accumulators are fp32; a weight enters the second product rounded to the
-// model dtype.
+// model dtype.  With key_splits > 1 (steps of short runs over long contexts) the keys of a row tile
+// are shared out to that many workgroups, which leave their sums in scratch for a merge launch.
 template <class S>
 struct LatentMfma;
 template <>
@@ -215,20 +217,21 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     typename S::T* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride,
     LatentQuery<S> q, const typename S::T* __restrict__ cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
-    int heads, int rank, int rot, int block_size, int num_blocks, float scale, int hb, int tb) {
+    int heads, int rank, int rot, int block_size, int num_blocks, float scale, int hb, int tb,
+    int key_splits, float* __restrict__ part_o, float* __restrict__ part_ml, int num_tokens) {
   using T = typename S::T;
   using M = LatentMfma<S>;
   constexpr int WP = 2 * VBW + 2;                      // 16-byte pieces of a tile a thread stages
   extern __shared__ __align__(16) unsigned char smem[];
   const int width = rank + rot, row_elems = width + 8;   // rows stay 16-byte aligned
   const int row_pieces = width / 8, tile_pieces = kTileKeys * row_pieces;
-  T* q_lds = reinterpret_cast<T*>(smem);                                     // [32][row_elems]
-  T* k_lds2 = q_lds + kTileRows * row_elems;                                 // [2][32][row_elems]
-  float* s_lds = reinterpret_cast<float*>(k_lds2 + 2 * kTileKeys * row_elems);   // [4][4][64][4]
+  T* k_lds = reinterpret_cast<T*>(smem);                                     // [32][row_elems]
+  float* s_lds = reinterpret_cast<float*>(k_lds + kTileKeys * row_elems);    // [4][4][64][4]
   long long* rows_lds = reinterpret_cast<long long*>(s_lds + 4 * 16 * 64);   // [2][32]
   const int b = blockIdx.z;
   // the last tiles of a run have the most keys to walk: they are dispatched first
-  const int tile_x = gridDim.x - 1 - blockIdx.x;
+  const int flat_x = gridDim.x - 1 - blockIdx.x;
+  const int tile_x = flat_x / key_splits, split = flat_x - tile_x * key_splits;
   const int run = query_start_loc[b + 1] - query_start_loc[b];
   const int tq0 = tile_x * tb;
   if (tq0 >= run) return;
@@ -237,24 +240,30 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int hf = lane >> 5, c = lane & 31;
   const int t_first = query_start_loc[b] + tq0;
-  const int p_first = context_lens[b] + tq0, p_last = p_first + ntok - 1;
+  const int p_first = context_lens[b] + tq0, p_end = p_first + ntok - 1;
+  // this workgroup's share of the keys 0 .. p_end: whole tiles, the last share may be short or empty
+  const int share = ((p_end + key_splits) / key_splits + kTileKeys - 1) / kTileKeys * kTileKeys;
+  const int j_begin = split * share;
+  const int p_last = min(p_end, j_begin + share - 1);      // the last key this workgroup reads
   const int my_tok = c / hb, my_head = c - my_tok * hb;
   const bool my_row = my_tok < ntok && my_head < nh;
   const int pq = p_first + my_tok;
   const int* table = block_tables + (int64_t)b * max_blocks;
   const float scale2 = scale * 1.4426950408889634f;    // scores in base 2
 
-  for (int i = tid; i < kTileRows * row_pieces; i += 256) {
-    const int r = i / row_pieces, v = i - r * row_pieces;
-    const int tok = r / hb, hd = r - tok * hb;
+  // the query rows stay in registers: a wave keeps the k-steps w, w + 4, ... of the first product
+  const int ksteps = width / 16, vb = rank / 32;
+  u32x4 qf[WP];
+#pragma unroll
+  for (int u = 0; u < WP; ++u) {
+    const int d = 16 * (w + 4 * u) + 8 * hf;
     u32x4 val = {0u, 0u, 0u, 0u};
-    if (tok < ntok && hd < nh) {
-      const int64_t t = t_first + tok, h = h0 + hd;
-      val = 8 * v < rank
-                ? *reinterpret_cast<const u32x4*>(q.lat + t * q.lat_token_stride + h * q.lat_head_stride + 8 * v)
-                : *reinterpret_cast<const u32x4*>(q.rot + t * q.rot_token_stride + h * q.rot_head_stride + 8 * v - rank);
+    if (my_row && d < width) {
+      const int64_t t = t_first + my_tok, h = h0 + my_head;
+      val = d < rank ? *reinterpret_cast<const u32x4*>(q.lat + t * q.lat_token_stride + h * q.lat_head_stride + d)
+                     : *reinterpret_cast<const u32x4*>(q.rot + t * q.rot_token_stride + h * q.rot_head_stride + d - rank);
     }
-    *reinterpret_cast<u32x4*>(q_lds + r * row_elems + 8 * v) = val;
+    qf[u] = val;
   }
   f32x16 o[VBW];
 #pragma unroll
@@ -277,59 +286,65 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     const int j = j0 + tid;
     rows_lds[buf * kTileKeys + tid] = blk < 0 ? -1 : (long long)blk * block_size + j % block_size;
   };
+  // where this thread's pieces of a tile sit: key row of the tile, offset in the cache row, offset
+  // in the LDS tile (the same for every tile, so the divisions are done once)
   u32x4 stage[WP];
+  int piece_row[WP], piece_src[WP], piece_dst[WP];
+#pragma unroll
+  for (int u = 0; u < WP; ++u) {
+    const int i = tid + 256 * u;
+    const int r = i / row_pieces, v = i - r * row_pieces;
+    piece_row[u] = i < tile_pieces ? r : -1;
+    piece_src[u] = 8 * v;
+    piece_dst[u] = r * row_elems + 8 * v;
+  }
   auto fetch = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < WP; ++u) {
-      const int i = tid + 256 * u;
       u32x4 got = {0u, 0u, 0u, 0u};
-      if (i < tile_pieces) {
-        const int r = i / row_pieces, v = i - r * row_pieces;
-        const long long row = rows_lds[buf * kTileKeys + r];
-        if (row >= 0) got = *reinterpret_cast<const u32x4*>(cache + row * width + 8 * v);
+      if (piece_row[u] >= 0) {
+        const long long row = rows_lds[buf * kTileKeys + piece_row[u]];
+        if (row >= 0) got = *reinterpret_cast<const u32x4*>(cache + row * width + piece_src[u]);
       }
       stage[u] = got;
     }
   };
-  auto land = [&](int buf) {
+  auto land = [&]() {
 #pragma unroll
-    for (int u = 0; u < WP; ++u) {
-      const int i = tid + 256 * u;
-      if (i < tile_pieces) {
-        const int r = i / row_pieces, v = i - r * row_pieces;
-        *reinterpret_cast<u32x4*>(k_lds2 + (buf * kTileKeys + r) * row_elems + 8 * v) = stage[u];
-      }
-    }
+    for (int u = 0; u < WP; ++u)
+      if (piece_row[u] >= 0)
+        *reinterpret_cast<u32x4*>(k_lds + piece_dst[u]) = stage[u];
   };
-  // One barrier pair per tile.  At the top of step `it`: tile `it` is in LDS buffer it & 1, tile
-  // it + 1 in the staging registers, the rows of tile it + 2 in rows_lds[it & 1], and threads
-  // 0 .. 31 hold the block ids of tile it + 3.
+  // Three barriers per tile (two workgroups share a CU and fill each other's waits).  At the top of
+  // step `it`: tile `it` is in LDS, tile it + 1 in the staging registers, the rows of tile it + 2
+  // in rows_lds[it & 1], and threads 0 .. 31 hold the block ids of tile it + 3.
   int blk_next = -1;
   if (tid < kTileKeys) {
-    store_row(0, load_block(0), 0);
-    store_row(kTileKeys, load_block(kTileKeys), 1);
+    store_row(j_begin, load_block(j_begin), 0);
+    store_row(j_begin + kTileKeys, load_block(j_begin + kTileKeys), 1);
   }
   __syncthreads();
   fetch(0);
-  land(0);
+  land();
   fetch(1);
   __syncthreads();
   if (tid < kTileKeys) {
-    store_row(2 * kTileKeys, load_block(2 * kTileKeys), 0);
-    blk_next = load_block(3 * kTileKeys);
+    store_row(j_begin + 2 * kTileKeys, load_block(j_begin + 2 * kTileKeys), 0);
+    blk_next = load_block(j_begin + 3 * kTileKeys);
   }
   __syncthreads();
-  const int ksteps = width / 16, vb = rank / 32;
   int it = 0;
-  for (int j0 = 0; j0 <= p_last; j0 += kTileKeys, ++it) {
-    const T* k_lds = k_lds2 + (it & 1) * kTileKeys * row_elems;
+  for (int j0 = j_begin; j0 <= p_last; j0 += kTileKeys, ++it) {
     f32x16 st;
 #pragma unroll
     for (int i = 0; i < 16; ++i) st[i] = 0.f;
-    for (int ks = w; ks < ksteps; ks += 4) {
-      const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + c * row_elems + 16 * ks + 8 * hf);
-      const u32x4 bq = *reinterpret_cast<const u32x4*>(q_lds + c * row_elems + 16 * ks + 8 * hf);
-      st = M::run(a, bq, st);
+#pragma unroll
+    for (int u = 0; u < WP; ++u) {
+      const int ks = w + 4 * u;
+      if (ks < ksteps) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(k_lds + c * row_elems + 16 * ks + 8 * hf);
+        st = M::run(a, qf[u], st);
+      }
     }
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
@@ -397,7 +412,8 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
         }
       }
     }
-    if (j0 + kTileKeys <= p_last) land((it + 1) & 1);            // tile it + 1, fetched a step ago
+    __syncthreads();                                             // everyone is done with tile it
+    if (j0 + kTileKeys <= p_last) land();                        // tile it + 1, fetched a step ago
     if (j0 + 2 * kTileKeys <= p_last) fetch(it & 1);             // tile it + 2 on its way
     if (tid < kTileKeys && j0 + 3 * kTileKeys <= p_last) {
       store_row(j0 + 3 * kTileKeys, blk_next, (it + 1) & 1);
@@ -407,6 +423,23 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
   }
   l += __shfl_xor(l, 32, 64);
   if (!my_row) return;
+  if (key_splits > 1) {
+    // this share's sums, not normalized, with the wave's own max and sum beside them
+    const int64_t row = ((int64_t)split * num_tokens + t_first + my_tok) * heads + h0 + my_head;
+    if (hf == 0) {
+      part_ml[(row * 4 + w) * 2] = m;
+      part_ml[(row * 4 + w) * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int n = 0; n < VBW; ++n) {
+      const int blk = w + 4 * n;
+      if (blk < vb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) part_o[row * rank + 32 * blk + (i & 3) + 8 * (i >> 2) + 4 * hf] = o[n][i];
+      }
+    }
+    return;
+  }
   const float inv = 1.f / l;
   T* orow = out + (int64_t)(t_first + my_tok) * out_token_stride + (int64_t)(h0 + my_head) * out_head_stride;
 #pragma unroll
@@ -417,6 +450,36 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
       for (int i = 0; i < 16; ++i)
         orow[32 * blk + (i & 3) + 8 * (i >> 2) + 4 * hf] = S::from_f32(o[n][i] * inv);
     }
+  }
+}
+
+// out[t, h, d] = sum_s o_s[d] 2^(m_s - M) / sum_s l_s 2^(m_s - M) over the key shares s, M the
+// largest m_s; the block of 32 dims d belongs to wave (d / 32) % 4 of the shares' workgroups
+template <class S>
+__global__ __launch_bounds__(256) void latent_merge_kernel(
+    typename S::T* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride,
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, int key_splits,
+    int num_tokens, int heads, int rank) {
+  const int64_t th = blockIdx.x;                 // token * heads + head
+  const int64_t t = th / heads;
+  const int h = (int)(th - t * heads);
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    const int w = (d >> 5) & 3;
+    const int64_t stride = (int64_t)num_tokens * heads;        // rows between two shares
+    const float* ml = part_ml + ((t * heads + h) * 4 + w) * 2;
+    const float* po = part_o + (t * heads + h) * rank + d;
+    float big = -INFINITY;
+#pragma unroll 8
+    for (int sp = 0; sp < key_splits; ++sp) big = fmaxf(big, ml[sp * stride * 8]);
+    float num = 0.f, den = 0.f;
+#pragma unroll 8
+    for (int sp = 0; sp < key_splits; ++sp) {
+      const float ms = ml[sp * stride * 8], ls = ml[sp * stride * 8 + 1], ov = po[sp * stride * rank];
+      const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - big);   // an empty share
+      num += ov * f;
+      den += ls * f;
+    }
+    out[t * out_token_stride + h * out_head_stride + d] = S::from_f32(num / den);
   }
 }
 
@@ -433,7 +496,8 @@ int launch_latent_tiles(dim3 grid, size_t lds, hipStream_t stream, typename S::T
                         int64_t out_token_stride, int64_t out_head_stride, const LatentQuery<S>& q,
                         const typename S::T* cache, const int* block_tables, int max_blocks,
                         const int* qsl, const int* ctx, int heads, int rank, int rot, int block_size,
-                        int num_blocks, float scale, int hb, int tb) {
+                        int num_blocks, float scale, int hb, int tb, int key_splits, float* part_o,
+                        float* part_ml, int num_tokens) {
   static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
   if (lds > allowed.load(std::memory_order_relaxed)) {
     VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
@@ -443,8 +507,13 @@ int launch_latent_tiles(dim3 grid, size_t lds, hipStream_t stream, typename S::T
   }
   latent_attention_tile_kernel<S, VBW><<<grid, 256, lds, stream>>>(
       out, out_token_stride, out_head_stride, q, cache, block_tables, max_blocks, qsl, ctx, heads,
-      rank, rot, block_size, num_blocks, scale, hb, tb);
+      rank, rot, block_size, num_blocks, scale, hb, tb, key_splits, part_o, part_ml, num_tokens);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
+  if (key_splits > 1) {
+    latent_merge_kernel<S><<<(unsigned)((int64_t)num_tokens * heads), 256, 0, stream>>>(
+        out, out_token_stride, out_head_stride, part_o, part_ml, key_splits, num_tokens, heads, rank);
+    VLA_SEQ_HIP_CHECK(hipGetLastError());
+  }
   return VLA_OK;
 }
 
@@ -523,16 +592,23 @@ extern "C" int vla_seq_latent_attention_tiles_supported(int rank, int rot, int d
          g_latent_kernel.load(std::memory_order_relaxed) == 0;
 }
 
+extern "C" int64_t vla_seq_latent_attention_scratch_floats(int key_splits, int num_tokens, int heads,
+                                                           int rank) {
+  return key_splits > 1 ? (int64_t)key_splits * num_tokens * heads * (rank + 8) : 0;
+}
+
 extern "C" int vla_seq_latent_attention_tiles(
     void* out, int64_t out_token_stride, int64_t out_head_stride, const void* q_lat,
     int64_t lat_token_stride, int64_t lat_head_stride, const void* q_rot, int64_t rot_token_stride,
     int64_t rot_head_stride, const void* cache, const int* block_tables, int max_blocks,
     const int* query_start_loc, const int* context_lens, int num_seqs, int max_query_len, int heads,
-    int rank, int rot, int block_size, int num_blocks, float scale, int dtype, void* stream) {
+    int rank, int rot, int block_size, int num_blocks, float scale, int key_splits, float* scratch,
+    int num_tokens, int dtype, void* stream) {
   if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
   if (!out || !q_lat || (rot > 0 && !q_rot) || !cache || !block_tables || !query_start_loc ||
       !context_lens || num_seqs < 0 || num_seqs > 65535 || max_query_len < 0 || heads <= 0 ||
-      rot < 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0)
+      rot < 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0 || key_splits < 1 ||
+      key_splits > 64 || (key_splits > 1 && (!scratch || num_tokens <= 0)))
     return VLA_ERR_ARG;
   if ((dtype != VLA_F16 && dtype != VLA_BF16) || !latent_tile_sizes(rank, rot)) return VLA_ERR_HEAD_SIZE;
   // 16-byte fragment loads: query rows and cache rows must allow them
@@ -541,9 +617,12 @@ extern "C" int vla_seq_latent_attention_tiles(
     return VLA_ERR_ARG;
   const int hb = heads < kTileRows ? heads : kTileRows;     // heads of a workgroup's rows
   const int tb = kTileRows / hb;                            // tokens of a workgroup's rows
-  const dim3 grid((max_query_len + tb - 1) / tb, (heads + hb - 1) / hb, num_seqs);
+  const dim3 grid((max_query_len + tb - 1) / tb * key_splits, (heads + hb - 1) / hb, num_seqs);
+  // scratch: the shares' sums [key_splits, T, heads, rank], then their max / sum per wave
+  float* part_o = scratch;
+  float* part_ml = scratch ? scratch + (int64_t)key_splits * num_tokens * heads * rank : nullptr;
   const int row_elems = rank + rot + 8;
-  const size_t lds = (size_t)3 * kTileRows * row_elems * 2 + 4 * 16 * 64 * sizeof(float) +
+  const size_t lds = (size_t)kTileKeys * row_elems * 2 + 4 * 16 * 64 * sizeof(float) +
                      2 * kTileKeys * sizeof(long long);
   if (lds > 160 * 1024) return VLA_ERR_HEAD_SIZE;
   const int vbw = (rank / 32 + 3) / 4;
@@ -557,7 +636,8 @@ extern "C" int vla_seq_latent_attention_tiles(
     return launch_latent_tiles<S, N>(grid, lds, (hipStream_t)stream, (T*)out, out_token_stride,     \
                                      out_head_stride, q, (const T*)cache, block_tables, max_blocks, \
                                      query_start_loc, context_lens, heads, rank, rot, block_size,   \
-                                     num_blocks, scale, hb, tb);
+                                     num_blocks, scale, hb, tb, key_splits, part_o, part_ml,        \
+                                     num_tokens);
     switch (vbw) {
       VLA_LATENT_CASE(1)
       VLA_LATENT_CASE(2)
