@@ -48,6 +48,9 @@ def configs():
         # more taps than some requests have tokens
         "taps": R.make_config([G(32, 2, conv=6, mlp=M(48)), D(2, 1, 32, conv=7, mlp=E(4, 2, 16)),
                                A(2, 32, 16, 32, 32, 24, scaling=YARN, mlp=None)], width=48),
+        # nothing a multiple of eight: widths, ranks, head sizes, vocabulary, the side input's size
+        "ragged": R.make_config([A(3, 10, 6, 14, 10, 18, scaling=YARN, mlp=E(5, 2, 18)), D(3, 3, 12, vdim=10, conv=3, mlp=M(50)),
+                                 G(30, 3, conv=5, mlp=E(4, 4, 6))], vocab=101, width=44, side_dim=5),
         # sizes for the matrix-core kernels: multiples of 32, many heads
         "mfma": R.make_config([A(10, 32, 32, 32, 64, 48, scaling=YARN, mlp=M(64)), D(4, 2, 32, vdim=64, mlp=E(6, 2, 32)),
                                A(3, 64, 64, 32, 96, 64, mlp=None)], width=128),
@@ -472,7 +475,7 @@ def test_whole_prompt_portions_and_decoding_agree_with_the_reference(tmp_path, n
         within(logit_error(run(sizes, sid), want), dtype, sid)
 
 
-@pytest.mark.parametrize("name", ["plain", "odd", "equal"])
+@pytest.mark.parametrize("name", ["plain", "odd", "equal", "ragged"])
 def test_layer_by_layer_against_the_reference(tmp_path, name):
     """The stream after every layer, float32."""
     s = Served(tmp_path, name, torch.float32)
