@@ -247,6 +247,7 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
   const int p_last = min(p_end, j_begin + share - 1);      // the last key this workgroup reads
   const int my_tok = c / hb, my_head = c - my_tok * hb;
   const bool my_row = my_tok < ntok && my_head < nh;
+  const bool all_rows = ntok * hb == kTileRows && nh == hb;    // no idle row in this workgroup
   const int pq = p_first + my_tok;
   const int* table = block_tables + (int64_t)b * max_blocks;
   const float scale2 = scale * 1.4426950408889634f;    // scores in base 2
@@ -284,7 +285,8 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
   };
   auto store_row = [&](int j0, int blk, int buf) {
     const int j = j0 + tid;
-    rows_lds[buf * kTileKeys + tid] = blk < 0 ? -1 : (long long)blk * block_size + j % block_size;
+    // the row's first element in the cache, so that a fetch only adds its piece's offset
+    rows_lds[buf * kTileKeys + tid] = blk < 0 ? -1 : ((long long)blk * block_size + j % block_size) * width;
   };
   // where this thread's pieces of a tile sit: key row of the tile, offset in the cache row, offset
   // in the LDS tile (the same for every tile, so the divisions are done once)
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
       u32x4 got = {0u, 0u, 0u, 0u};
       if (piece_row[u] >= 0) {
         const long long row = rows_lds[buf * kTileKeys + piece_row[u]];
-        if (row >= 0) got = *reinterpret_cast<const u32x4*>(cache + row * width + piece_src[u]);
+        if (row >= 0) got = *reinterpret_cast<const u32x4*>(cache + row + piece_src[u]);
       }
       stage[u] = got;
     }
@@ -364,11 +366,16 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     }
     // (the sum above runs in a different order in each wave; every wave keeps its own max and sum, and
     // they only need to agree with its own weights)
+    // every key of the tile visible to every row of a full workgroup: no masks
+    const bool full = all_rows && j0 + kTileKeys - 1 <= p_first;
     float mt = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int j = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
-      const float v = my_row && j <= pq ? st[i] * scale2 : -INFINITY;
+      float v = st[i] * scale2;
+      if (!full) {
+        const int j = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+        v = my_row && j <= pq ? v : -INFINITY;
+      }
       st[i] = v;
       mt = fmaxf(mt, v);
     }
