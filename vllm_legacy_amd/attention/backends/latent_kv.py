@@ -76,7 +76,7 @@ class LatentKVAttention(nn.Module):
         self.latent_norm.data = latent_norm.float().to(dev).contiguous()
 
     # workgroups a launch should have before the keys of a row tile stay with one workgroup
-    SPLIT_BELOW_WORKGROUPS = 1024
+    SPLIT_BELOW_WORKGROUPS = 512
     KEYS_PER_SPLIT = 256
 
     def key_splits(self, batch: SequenceBatch) -> int:
