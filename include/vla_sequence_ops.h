@@ -167,6 +167,24 @@ int vla_seq_gated_act(void* out, int64_t out_stride, const void* gate, int64_t g
                       const void* up, int64_t up_stride, int num_tokens, int features, int act,
                       int dtype, void* stream);
 
+/* out = g * sigmoid(alpha g) * (u + shift) with g = min(gate, limit), u = clamp(up, -limit, limit);
+ * rows of `features` values with their own strides, fp32 arithmetic. */
+int vla_seq_clamped_glu(void* out, int64_t out_stride, const void* gate, int64_t gate_stride,
+                        const void* up, int64_t up_stride, int num_tokens, int features, float limit,
+                        float alpha, float shift, int dtype, void* stream);
+
+/* out[t] (fp32 [T, width]) = table[ids[t]] + pair_table[r], r = (prev * mul_prev + ids[t] * mul_cur)
+ * mod buckets with prev the token before t in its sequence, r = buckets for a sequence's first
+ * token (pair_table has buckets + 1 rows).  The token before a step's first row is read from
+ * last_token[state_slots[b]] (int64 [num_slots]) when context_lens[b] > 0; afterwards every
+ * sequence's slot receives its last token of the step. */
+int vla_seq_pair_hash_embed(float* out, const void* table, const void* pair_table,
+                            const int64_t* ids, int64_t* last_token, const int* query_start_loc,
+                            const int* context_lens, const int* state_slots, const int* token_seq,
+                            int num_tokens, int num_seqs, int num_slots, int width, int vocab,
+                            int64_t buckets, int64_t mul_prev, int64_t mul_cur, int dtype,
+                            void* stream);
+
 /* ---- attention over paged key and value caches with rotary positions ------------------------- */
 
 /* Rotates the step's queries in place and writes its rotated keys and values to the caches
@@ -175,17 +193,25 @@ int vla_seq_gated_act(void* out, int64_t out_stride, const void* gate, int64_t g
  * (i, i + rot_dims / 2) otherwise -- turns by positions[t] * inv_freq[i]: (a, b) ->
  * (a cos - b sin, b cos + a sin).  value_inv_freq [vdim / 2] (null: values are cached as they
  * are) turns the pairs of a value head over all vdim elements the same way.  Angles are fp32
- * products.  slot_mapping < 0 skips the caches. */
+ * products.  slot_mapping < 0 skips the caches.  q_norm [heads * dim] / k_norm [kv_heads * dim]
+ * (fp32, null: none): the whole query / key row is divided by its root mean square (norm_eps inside
+ * the root) and multiplied by these weights before it is rotated.  v_other (null: none; rows of
+ * kv_heads * vdim values, not together with value_inv_freq): the cached value is
+ * (1 - v_blend[0]) v + v_blend[0] v_other, v_blend one fp32 number on the device. */
 int vla_seq_rotary_kv_write(void* q, int64_t q_stride, const void* k, int64_t k_stride,
                             const void* v, int64_t v_stride, void* key_cache, void* value_cache,
                             const int64_t* positions, const int64_t* slot_mapping,
                             const float* inv_freq, const float* value_inv_freq, int num_tokens,
                             int heads, int kv_heads, int dim, int vdim, int rot_dims,
                             int interleaved, int block_size, int num_blocks, int dtype,
+                            const float* q_norm, const float* k_norm, float norm_eps,
+                            const void* v_other, int64_t v_other_stride, const float* v_blend,
                             void* stream);
 
 /* For the token at position p of sequence b and query head h (KV head h / (heads / kv_heads)):
  *   s_j = (q . k_j) * scale  for max(0, p - window + 1) <= j <= p  (window <= 0: all j <= p)
+ *         and, with a window, for j < keep_first as well (a sequence's first tokens stay visible)
+ *   s_j <- softcap * tanh(s_j / softcap)                      (softcap 0: no cap)
  *   o = sum_j softmax(s)_j v_j;  out_inv_freq given: pair m of o turns by -p * out_inv_freq[m]
  *   out = dtype(o * sigmoid(gate[t, h]))                      (gate null: no gate)
  * in fp32; the step's own keys and values must be in the caches already.  gate holds one number
@@ -196,7 +222,7 @@ int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q, int64_t q
                          const int* token_seq, const int64_t* positions, const float* out_inv_freq,
                          int interleaved, int num_tokens, int heads, int kv_heads, int dim, int vdim,
                          int block_size, int num_blocks, int window, float scale, int dtype,
-                         void* stream);
+                         int keep_first, float softcap, void* stream);
 
 /* The same attention for 16-bit activations, tiled over runs of 32 query rows of a sequence on
  * the matrix cores: rows query_start_loc[b] .. query_start_loc[b + 1] - 1 of sequence b sit at
@@ -212,7 +238,7 @@ int vla_seq_kv_attention_tiles(void* out, int64_t out_stride, const void* q, int
                                const float* out_inv_freq, int interleaved, int num_seqs,
                                int max_query_len, int heads, int kv_heads, int dim, int vdim,
                                int block_size, int num_blocks, int window, float scale, int dtype,
-                               void* stream);
+                               int keep_first, float softcap, void* stream);
 int vla_seq_set_kv_attention_kernel(int mode);
 
 /* ---- element-wise gated recurrence (minGRU) ---------------------------------------------------- */
@@ -359,8 +385,9 @@ int vla_seq_rglru_scan(void* out, int64_t out_stride, int out_dtype, const float
 
 /* cache [num_blocks, block_size, rank + rot] (`dtype`): per token the normed latent and the rotated
  * key part every head shares.  Rotates the rot_dims first elements of every head's rotated query
- * part in place (head h's part starts at q + t q_stride + h q_head_stride + q_first; interleaved
- * pairs (2i, 2i + 1) turn by positions[t] * inv_freq[i], sine and cosine times `magnitude`) and
+ * part in place (head h's part starts at q + t q_stride + h q_head_stride + q_first; pairs
+ * (2i, 2i + 1) when interleaved, (i, i + rot_dims / 2) otherwise, turn by positions[t] * inv_freq[i],
+ * sine and cosine times `magnitude`) and
  * writes the rows [kv[:rank] / sqrt(mean^2 + eps) * norm_weight | kv[rank:] rotated the same way].
  * slot_mapping < 0 skips the cache. */
 int vla_seq_latent_rotary_write(void* q, int64_t q_stride, int q_head_stride, int q_first,
@@ -368,18 +395,22 @@ int vla_seq_latent_rotary_write(void* q, int64_t q_stride, int q_head_stride, in
                                 float eps, void* cache, const int64_t* positions,
                                 const int64_t* slot_mapping, const float* inv_freq, float magnitude,
                                 int num_tokens, int heads, int rank, int rot, int rot_dims,
-                                int block_size, int num_blocks, int dtype, void* stream);
+                                int block_size, int num_blocks, int dtype, int interleaved,
+                                void* stream);
 
 /* out[t, h, :rank] = sum_j p_j c_j over the keys j <= position of the row's sequence, p = softmax
  * of (q_lat[t, h] . c_j + q_rot[t, h] . k_rot_j) * scale; q_lat, q_rot and out are addressed by a
- * token stride and a head stride each.  Any dtype, rank and rot up to 1024. */
+ * token stride and a head stride each.  window > 0 keeps the keys with position - j < window only;
+ * gate (null: none; one number per (token, head), row stride gate_stride) multiplies a head's sums
+ * by its sigmoid.  Any dtype, rank and rot up to 1024. */
 int vla_seq_latent_attention(void* out, int64_t out_token_stride, int64_t out_head_stride,
                              const void* q_lat, int64_t lat_token_stride, int64_t lat_head_stride,
                              const void* q_rot, int64_t rot_token_stride, int64_t rot_head_stride,
                              const void* cache, const int* block_tables, int max_blocks,
                              const int* token_seq, const int64_t* positions, int num_tokens,
                              int heads, int rank, int rot, int block_size, int num_blocks,
-                             float scale, int dtype, void* stream);
+                             float scale, int dtype, int window, const void* gate,
+                             int64_t gate_stride, void* stream);
 
 /* The same attention on the matrix cores for 16-bit models: 32 query rows that are (token, head)
  * pairs of one sequence per workgroup, tiles of 32 keys.  rank a multiple of 32 up to 512, rot a
@@ -399,7 +430,8 @@ int vla_seq_latent_attention_tiles(void* out, int64_t out_token_stride, int64_t 
                                    const int* query_start_loc, const int* context_lens,
                                    int num_seqs, int max_query_len, int heads, int rank, int rot,
                                    int block_size, int num_blocks, float scale, int key_splits,
-                                   float* scratch, int num_tokens, int dtype, void* stream);
+                                   float* scratch, int num_tokens, int dtype, int window,
+                                   const void* gate, int64_t gate_stride, void* stream);
 int vla_seq_set_latent_attention_kernel(int mode);
 
 /* Kernel choice for tests: window attention 0 = per shape, 1 = one wave per (row, head);

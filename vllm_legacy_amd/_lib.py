@@ -64,6 +64,7 @@ SEQ_EXPORTS = [
     "vla_seq_embed_scaled", "vla_seq_softcap", "vla_seq_delta_rule_scan", "vla_seq_delta_rule_scratch_floats", "vla_seq_set_delta_kernel", "vla_seq_rglru_scan",
     "vla_seq_latent_rotary_write", "vla_seq_latent_attention", "vla_seq_latent_attention_tiles",
     "vla_seq_latent_attention_tiles_supported", "vla_seq_latent_attention_scratch_floats", "vla_seq_set_latent_attention_kernel",
+    "vla_seq_clamped_glu", "vla_seq_pair_hash_embed",
 ]
 _seq_lib = None
 
@@ -111,12 +112,12 @@ def seq_lib():
         L.vla_seq_concat_cast.argtypes = [p, p, p, i, i, i, p]
         L.vla_seq_gated_act.argtypes = [p, i64, p, i64, p, i64, i, i, i, i, p]
         L.vla_seq_rotary_kv_write.argtypes = [p, i64, p, i64, p, i64, p, p, p, p, p, p, i, i, i, i, i,
-                                              i, i, i, i, i, p]
+                                              i, i, i, i, i, p, p, f, p, i64, p, p]
         L.vla_seq_kv_attention.argtypes = [p, i64, p, i64, p, i64, p, p, p, i, p, p, p, i, i, i, i, i,
-                                           i, i, i, i, f, i, p]
+                                           i, i, i, i, f, i, i, f, p]
         L.vla_seq_kv_attention_tiles_supported.argtypes = [i, i, i]
         L.vla_seq_kv_attention_tiles.argtypes = [p, i64, p, i64, p, i64, p, p, p, i, p, p, p, i, i, i,
-                                                 i, i, i, i, i, i, i, f, i, p]
+                                                 i, i, i, i, i, i, i, f, i, i, f, p]
         L.vla_seq_set_kv_attention_kernel.argtypes = [i]
         L.vla_seq_set_grouped_linear_form.argtypes = [i]
         L.vla_seq_mingru_scratch_floats.argtypes = [i, i, i]
@@ -138,16 +139,18 @@ def seq_lib():
         L.vla_seq_rglru_scan.argtypes = [p, i64, i, p, i64, p, i64, i, i64, p, i64, p, i64, p, p, p, p, p, i, i,
                                          i, i, p, i64, p]
         L.vla_seq_latent_rotary_write.argtypes = [p, i64, i, i, p, i64, p, f, p, p, p, p, f, i, i, i, i, i,
-                                                  i, i, i, p]
+                                                  i, i, i, i, p]
         L.vla_seq_latent_attention.argtypes = [p, i64, i64, p, i64, i64, p, i64, i64, p, p, i, p, p, i, i,
-                                               i, i, i, i, f, i, p]
+                                               i, i, i, i, f, i, i, p, i64, p]
         L.vla_seq_moe_tile_rows.argtypes = []
         L.vla_seq_moe_plan.argtypes = [p, i, i, i, p, p, p, i, p]
         L.vla_seq_grouped_linear.argtypes = [p, i64, i, p, i64, p, p, p, i, i, i, i, i, p]
         L.vla_seq_moe_combine.argtypes = [p, p, p, p, p, i64, p, p, i, i, i, i, p]
         L.vla_seq_latent_attention_tiles_supported.argtypes = [i, i, i]
         L.vla_seq_latent_attention_tiles.argtypes = [p, i64, i64, p, i64, i64, p, i64, i64, p, p, i, p, p, i, i,
-                                                     i, i, i, i, i, f, i, p, i, i, p]
+                                                     i, i, i, i, i, f, i, p, i, i, i, p, i64, p]
+        L.vla_seq_clamped_glu.argtypes = [p, i64, p, i64, p, i64, i, i, f, f, f, i, p]
+        L.vla_seq_pair_hash_embed.argtypes = [p, p, p, p, p, p, p, p, p, i, i, i, i, i, i64, i64, i64, i, p]
         L.vla_seq_latent_attention_scratch_floats.argtypes = [i, i, i, i]
         L.vla_seq_latent_attention_scratch_floats.restype = i64
         L.vla_seq_set_latent_attention_kernel.argtypes = [i]

@@ -331,13 +331,56 @@ def gated_act(out: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor],
             0 if up is None else _rows(up, F), T, F, ACT[act], _dt(gate.dtype), _stream(gate.device)), "gated_act")
 
 
+def clamped_glu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, limit: float, alpha: float,
+                shift: float) -> None:
+    """out = g * sigmoid(alpha g) * (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit);
+    [T, F] views with free row strides."""
+    _gpu(out, gate, up)
+    T, F = gate.shape
+    assert out.shape == gate.shape == up.shape and out.dtype == gate.dtype == up.dtype
+    with torch.cuda.device(gate.device):
+        seq_check(_lib.seq_lib().vla_seq_clamped_glu(
+            out.data_ptr(), _rows(out, F), gate.data_ptr(), _rows(gate, F), up.data_ptr(), _rows(up, F), T, F,
+            float(limit), float(alpha), float(shift), _dt(gate.dtype), _stream(gate.device)), "clamped_glu")
+
+
+def pair_hash_embed(out: torch.Tensor, table: torch.Tensor, pair_table: torch.Tensor, ids: torch.Tensor,
+                    last_token: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
+                    state_slots: torch.Tensor, token_seq: torch.Tensor, mul_prev: int, mul_cur: int) -> None:
+    """out fp32 [T, W] = table[ids] + pair_table[(prev * mul_prev + id * mul_cur) mod buckets], the
+    table's last row (number buckets) for a sequence's first token; last_token int64 [slots] holds
+    every sequence's last token between steps and is brought up to date."""
+    _gpu(out, table, pair_table, ids, last_token, query_start_loc, context_lens, state_slots, token_seq)
+    T, W = out.shape
+    B = context_lens.numel()
+    assert out.dtype == torch.float32 and out.is_contiguous()
+    assert table.is_contiguous() and pair_table.is_contiguous() and table.dtype == pair_table.dtype
+    assert table.shape[1] == W and pair_table.shape[1] == W and pair_table.shape[0] >= 2
+    assert ids.dtype == torch.int64 and ids.numel() == T and ids.is_contiguous()
+    assert last_token.dtype == torch.int64 and last_token.is_contiguous() and last_token.dim() == 1
+    for t in (query_start_loc, context_lens, state_slots, token_seq):
+        assert t.dtype == torch.int32 and t.is_contiguous()
+    assert query_start_loc.numel() == B + 1 and state_slots.numel() == B and token_seq.numel() == T
+    with torch.cuda.device(out.device):
+        seq_check(_lib.seq_lib().vla_seq_pair_hash_embed(
+            out.data_ptr(), table.data_ptr(), pair_table.data_ptr(), ids.data_ptr(), last_token.data_ptr(),
+            query_start_loc.data_ptr(), context_lens.data_ptr(), state_slots.data_ptr(), token_seq.data_ptr(), T, B,
+            last_token.numel(), W, table.shape[0], pair_table.shape[0] - 1, int(mul_prev), int(mul_cur),
+            _dt(table.dtype), _stream(out.device)), "pair_hash_embed")
+
+
 def rotary_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_cache: torch.Tensor,
                     value_cache: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
                     inv_freq: Optional[torch.Tensor], value_inv_freq: Optional[torch.Tensor], heads: int,
-                    rot_dims: int, interleaved: bool) -> None:
+                    rot_dims: int, interleaved: bool, q_norm: Optional[torch.Tensor] = None,
+                    k_norm: Optional[torch.Tensor] = None, norm_eps: float = 0.0,
+                    v_other: Optional[torch.Tensor] = None, v_blend: Optional[torch.Tensor] = None) -> None:
     """q [T, H*D] rotated in place; k [T, G*D], v [T, G*V] rotated into the caches
-    [NB, BS, G, D] / [NB, BS, G, V]."""
-    _gpu(q, k, v, key_cache, value_cache, positions, slot_mapping, inv_freq, value_inv_freq)
+    [NB, BS, G, D] / [NB, BS, G, V].  q_norm fp32 [H*D] / k_norm fp32 [G*D]: the whole query / key
+    row is RMS-normed with these weights before the rotation.  v_other [T, G*V] with v_blend (fp32,
+    one number on the device): the cached value is (1 - v_blend) v + v_blend v_other."""
+    _gpu(q, k, v, key_cache, value_cache, positions, slot_mapping, inv_freq, value_inv_freq, q_norm, k_norm,
+         v_other, v_blend)
     NB, BS, G, D = key_cache.shape
     V = value_cache.shape[3]
     T = q.shape[0]
@@ -349,20 +392,27 @@ def rotary_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, key_cache
         assert inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2 and inv_freq.is_contiguous()
     if value_inv_freq is not None:
         assert value_inv_freq.dtype == torch.float32 and value_inv_freq.numel() == V // 2
+    assert q_norm is None or (q_norm.dtype == torch.float32 and q_norm.numel() == heads * D and q_norm.is_contiguous())
+    assert k_norm is None or (k_norm.dtype == torch.float32 and k_norm.numel() == G * D and k_norm.is_contiguous())
+    if v_other is not None:
+        assert v_other.dtype == v.dtype and v_other.shape == v.shape and value_inv_freq is None
+        assert v_blend is not None and v_blend.dtype == torch.float32 and v_blend.numel() == 1
     with torch.cuda.device(q.device):
         seq_check(_lib.seq_lib().vla_seq_rotary_kv_write(
             q.data_ptr(), _rows(q, heads * D), k.data_ptr(), _rows(k, G * D), v.data_ptr(), _rows(v, G * V),
             key_cache.data_ptr(), value_cache.data_ptr(), positions.data_ptr(), slot_mapping.data_ptr(),
             _p(inv_freq), _p(value_inv_freq), T, heads, G, D, V, int(rot_dims), int(bool(interleaved)), BS, NB,
-            _dt(q.dtype), _stream(q.device)), "rotary_kv_write")
+            _dt(q.dtype), _p(q_norm), _p(k_norm), float(norm_eps), _p(v_other),
+            0 if v_other is None else _rows(v_other, G * V), _p(v_blend), _stream(q.device)), "rotary_kv_write")
 
 
 def kv_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], key_cache: torch.Tensor,
                  value_cache: torch.Tensor, block_tables: torch.Tensor, token_seq: torch.Tensor,
                  positions: torch.Tensor, out_inv_freq: Optional[torch.Tensor], interleaved: bool, heads: int,
-                 window: int, scale: float) -> None:
+                 window: int, scale: float, keep_first: int = 0, softcap: float = 0.0) -> None:
     """out [T, H*V] = softmax attention of q [T, H*D] over the caches, output pairs turned back by
-    the position, times sigmoid(gate [T, H])."""
+    the position, times sigmoid(gate [T, H]).  With a window the first keep_first tokens of a
+    sequence stay visible; softcap > 0 caps the scores with softcap * tanh(score / softcap)."""
     _gpu(out, q, gate, key_cache, value_cache, block_tables, token_seq, positions, out_inv_freq)
     NB, BS, G, D = key_cache.shape
     V = value_cache.shape[3]
@@ -382,7 +432,7 @@ def kv_attention(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor
             0 if gate is None else _rows(gate, heads), key_cache.data_ptr(), value_cache.data_ptr(),
             block_tables.data_ptr(), block_tables.shape[1], token_seq.data_ptr(), positions.data_ptr(),
             _p(out_inv_freq), int(bool(interleaved)), T, heads, G, D, V, BS, NB, int(window), float(scale),
-            _dt(q.dtype), _stream(q.device)), "kv_attention")
+            _dt(q.dtype), int(keep_first), float(softcap), _stream(q.device)), "kv_attention")
 
 
 def set_kv_attention_kernel(mode: int) -> None:
@@ -399,7 +449,8 @@ def kv_attention_tiles_supported(q: torch.Tensor, head_dim: int, value_dim: int)
 def kv_attention_tiles(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.Tensor], key_cache: torch.Tensor,
                        value_cache: torch.Tensor, block_tables: torch.Tensor, query_start_loc: torch.Tensor,
                        context_lens: torch.Tensor, max_query_len: int, out_inv_freq: Optional[torch.Tensor],
-                       interleaved: bool, heads: int, window: int, scale: float) -> None:
+                       interleaved: bool, heads: int, window: int, scale: float, keep_first: int = 0,
+                       softcap: float = 0.0) -> None:
     """The same attention as kv_attention for 16-bit activations, tiled over runs of 32 query rows
     of a sequence."""
     _gpu(out, q, gate, key_cache, value_cache, block_tables, query_start_loc, context_lens, out_inv_freq)
@@ -421,7 +472,7 @@ def kv_attention_tiles(out: torch.Tensor, q: torch.Tensor, gate: Optional[torch.
             0 if gate is None else _rows(gate, heads), key_cache.data_ptr(), value_cache.data_ptr(),
             block_tables.data_ptr(), block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(),
             _p(out_inv_freq), int(bool(interleaved)), B, int(max_query_len), heads, G, D, V, BS, NB, int(window),
-            float(scale), _dt(q.dtype), _stream(q.device)), "kv_attention_tiles")
+            float(scale), _dt(q.dtype), int(keep_first), float(softcap), _stream(q.device)), "kv_attention_tiles")
 
 
 def mingru_scan(out: torch.Tensor, zp: torch.Tensor, up: torch.Tensor, gp: torch.Tensor, state: torch.Tensor,
@@ -687,7 +738,7 @@ def rglru_scan(out: torch.Tensor, gates: torch.Tensor, u: torch.Tensor, y: torch
 def latent_rotary_write(q: torch.Tensor, q_head_stride: int, q_first: int, heads: int, kv: torch.Tensor,
                         norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, positions: torch.Tensor,
                         slot_mapping: torch.Tensor, inv_freq: Optional[torch.Tensor], magnitude: float,
-                        rot_dims: int) -> None:
+                        rot_dims: int, interleaved: bool = True) -> None:
     """q [T, >= heads * q_head_stride]: the rotated part of head h starts at column h * q_head_stride +
     q_first; kv [T, rank + rot]; cache [NB, BS, rank + rot]."""
     _gpu(q, kv, norm_weight, cache, positions, slot_mapping, inv_freq)
@@ -707,15 +758,17 @@ def latent_rotary_write(q: torch.Tensor, q_head_stride: int, q_first: int, heads
             q.data_ptr(), q.stride(0) if T > 1 else q.shape[1], int(q_head_stride), int(q_first), kv.data_ptr(),
             _rows(kv, width), norm_weight.data_ptr(), float(eps), cache.data_ptr(), positions.data_ptr(),
             slot_mapping.data_ptr(), _p(inv_freq), float(magnitude), T, int(heads), rank, rot, int(rot_dims), BS, NB,
-            _dt(q.dtype), _stream(q.device)), "latent_rotary_write")
+            _dt(q.dtype), int(bool(interleaved)), _stream(q.device)), "latent_rotary_write")
 
 
 def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
                      block_tables: torch.Tensor, token_seq: torch.Tensor, positions: torch.Tensor,
-                     scale: float) -> None:
+                     scale: float, window: int = 0, gate: Optional[torch.Tensor] = None) -> None:
     """out, q_lat [T, H, rank] and q_rot [T, H, rot] views (any token / head strides, unit stride
-    along the last axis); cache [NB, BS, rank + rot]."""
-    _gpu(out, q_lat, q_rot, cache, block_tables, token_seq, positions)
+    along the last axis); cache [NB, BS, rank + rot]; window > 0: keys with position - j < window
+    only; gate [T, H]: a head's sums times sigmoid(gate)."""
+    _gpu(out, q_lat, q_rot, cache, block_tables, token_seq, positions, gate)
+    assert gate is None or gate.dtype == q_lat.dtype
     NB, BS, width = cache.shape
     T, H, rank = q_lat.shape
     rot = width - rank
@@ -731,7 +784,8 @@ def latent_attention(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor
             out.data_ptr(), out.stride(0), out.stride(1), q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1),
             q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1), cache.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], token_seq.data_ptr(), positions.data_ptr(), T, H, rank, rot, BS, NB, float(scale),
-            _dt(q_lat.dtype), _stream(q_lat.device)), "latent_attention")
+            _dt(q_lat.dtype), int(window), _p(gate), 0 if gate is None else _rows(gate, H),
+            _stream(q_lat.device)), "latent_attention")
 
 
 def set_latent_attention_kernel(mode: int) -> None:
@@ -752,15 +806,17 @@ def latent_attention_tiles_supported(q_lat: torch.Tensor, q_rot: torch.Tensor, c
 
 def latent_attention_tiles(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.Tensor, cache: torch.Tensor,
                            block_tables: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
-                           max_query_len: int, scale: float, key_splits: int = 1) -> None:
+                           max_query_len: int, scale: float, key_splits: int = 1, window: int = 0,
+                           gate: Optional[torch.Tensor] = None) -> None:
     """The same attention as latent_attention for 16-bit activations on the matrix cores; rows
     query_start_loc[b] .. of sequence b sit at positions context_lens[b] ...  key_splits > 1: the
     keys of every row tile are shared out to that many workgroups and merged."""
-    _gpu(out, q_lat, q_rot, cache, block_tables, query_start_loc, context_lens)
+    _gpu(out, q_lat, q_rot, cache, block_tables, query_start_loc, context_lens, gate)
     NB, BS, width = cache.shape
     T, H, rank = q_lat.shape
     rot = width - rank
     B = context_lens.numel()
+    assert gate is None or gate.dtype == q_lat.dtype
     assert out.shape == q_lat.shape and q_rot.shape == (T, H, rot) and cache.is_contiguous()
     assert out.dtype == q_lat.dtype == q_rot.dtype == cache.dtype
     for t in (out, q_lat, q_rot):
@@ -780,5 +836,6 @@ def latent_attention_tiles(out: torch.Tensor, q_lat: torch.Tensor, q_rot: torch.
             out.data_ptr(), st(out, 0), st(out, 1), q_lat.data_ptr(), st(q_lat, 0), st(q_lat, 1),
             q_rot.data_ptr(), st(q_rot, 0), st(q_rot, 1), cache.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], query_start_loc.data_ptr(), context_lens.data_ptr(), B, int(max_query_len), H, rank,
-            rot, BS, NB, float(scale), int(key_splits), _p(scratch), T, _dt(q_lat.dtype), _stream(q_lat.device)),
+            rot, BS, NB, float(scale), int(key_splits), _p(scratch), T, _dt(q_lat.dtype), int(window), _p(gate),
+            0 if gate is None else _rows(gate, H), _stream(q_lat.device)),
             "latent_attention_tiles")

@@ -1,7 +1,13 @@
 // Causal softmax attention over paged key and value caches with rotary positions on queries and
 // keys, values that are rotated by their own position when they are cached (the head's output is
-// turned back by the query's position), an optional sliding window and a sigmoid gate of one
-// number per head.
+// turned back by the query's position), an optional sliding window that may keep a sequence's
+// first tokens visible, an optional cap on the scores (cap * tanh(score / cap)) and a sigmoid gate of
+// one number per head.  rotary_kv_write can also norm the whole query and key rows before it rotates
+// them and blend the values with another layer's values of the same tokens.
+//
+// With a window and `keep_first` kept tokens, query position p sees j <= p with p - j < window or
+// j < keep_first.  The kernels walk such a key set through one index u: with lo the window's first
+// key and nk = min(keep_first, lo), u < nk is key u and u >= nk is key lo + u - nk.
 //
 // Caches: keys [num_blocks, block_size, kv_heads, dim] and values [num_blocks, block_size, kv_heads,
 // vdim] in the model dtype, token-major rows.  rotary_kv_write rotates the step's queries in place
@@ -34,6 +40,14 @@ __device__ __forceinline__ void turn(float& a, float& b, float angle) {
   a = a2;
 }
 
+// cap * tanh(s / cap): libm's tanh in the fp32 kernel, one exponential and one reciprocal in the
+// matrix-core kernels (absolute error of a few 1e-7 times cap)
+__device__ __forceinline__ float cap_score(float s, float cap) { return cap * tanhf(s / cap); }
+__device__ __forceinline__ float cap_score_fast(float s, float cap, float two_log2e_over_cap) {
+  const float e = __builtin_amdgcn_exp2f(s * two_log2e_over_cap);   // e^(2 s / cap); inf and 0 are fine
+  return cap - 2.f * cap * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
 // element indices of pair i among `span` rotated elements
 __device__ __forceinline__ void pair_index(int i, int span, int interleaved, int& ia, int& ib) {
   if (interleaved) {
@@ -53,42 +67,89 @@ __global__ __launch_bounds__(256) void rotary_kv_write_kernel(
     typename S::T* __restrict__ key_cache, typename S::T* __restrict__ value_cache,
     const int64_t* __restrict__ positions, const int64_t* __restrict__ slot_mapping,
     const float* __restrict__ inv_freq, const float* __restrict__ value_inv_freq, int heads,
-    int kv_heads, int dim, int vdim, int rot_dims, int interleaved, int64_t num_slots) {
+    int kv_heads, int dim, int vdim, int rot_dims, int interleaved, int64_t num_slots,
+    const float* __restrict__ q_norm, const float* __restrict__ k_norm, float norm_eps,
+    const typename S::T* __restrict__ v_other, int64_t v_other_stride,
+    const float* __restrict__ v_blend) {
   using T = typename S::T;
+  __shared__ float red[16];
   const int t = blockIdx.x;
   const float p = (float)positions[t];
   int64_t slot = slot_mapping[t];
   const bool cached = slot >= 0 && slot < num_slots;
   const int half = rot_dims / 2;
+  const int rest = dim - rot_dims;
   T* qr = q + (int64_t)t * q_stride;
+  const T* kr = k + (int64_t)t * k_stride;
+  // RMS norm over the whole row (all heads at once) with a weight per element, before the rotation
+  float q_inv = 1.f, k_inv = 1.f;
+  if (q_norm != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < heads * dim; i += blockDim.x) {
+      const float x = S::to_f32(qr[i]);
+      ss += x * x;
+    }
+    q_inv = 1.f / sqrtf(block_sum(ss, red) / (float)(heads * dim) + norm_eps);
+  }
+  if (k_norm != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
+      const float x = S::to_f32(kr[i]);
+      ss += x * x;
+    }
+    k_inv = 1.f / sqrtf(block_sum(ss, red) / (float)(kv_heads * dim) + norm_eps);
+  }
   for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
     const int h = i / half, f = i - h * half;
     int ia, ib;
     pair_index(f, rot_dims, interleaved, ia, ib);
     float a = S::to_f32(qr[h * dim + ia]), b = S::to_f32(qr[h * dim + ib]);
+    if (q_norm != nullptr) {
+      a *= q_inv * q_norm[h * dim + ia];
+      b *= q_inv * q_norm[h * dim + ib];
+    }
     turn(a, b, p * inv_freq[f]);
     qr[h * dim + ia] = S::from_f32(a);
     qr[h * dim + ib] = S::from_f32(b);
   }
+  if (q_norm != nullptr) {
+    for (int i = threadIdx.x; i < heads * rest; i += blockDim.x) {
+      const int h = i / rest, d = rot_dims + (i - h * rest);
+      qr[h * dim + d] = S::from_f32(S::to_f32(qr[h * dim + d]) * q_inv * q_norm[h * dim + d]);
+    }
+  }
   if (!cached) return;
-  const T* kr = k + (int64_t)t * k_stride;
   T* kc = key_cache + slot * (int64_t)kv_heads * dim;
   for (int i = threadIdx.x; i < kv_heads * half; i += blockDim.x) {
     const int h = i / half, f = i - h * half;
     int ia, ib;
     pair_index(f, rot_dims, interleaved, ia, ib);
     float a = S::to_f32(kr[h * dim + ia]), b = S::to_f32(kr[h * dim + ib]);
+    if (k_norm != nullptr) {
+      a *= k_inv * k_norm[h * dim + ia];
+      b *= k_inv * k_norm[h * dim + ib];
+    }
     turn(a, b, p * inv_freq[f]);
     kc[h * dim + ia] = S::from_f32(a);
     kc[h * dim + ib] = S::from_f32(b);
   }
-  const int rest = dim - rot_dims;
   for (int i = threadIdx.x; i < kv_heads * rest; i += blockDim.x) {
     const int h = i / rest, d = rot_dims + (i - h * rest);
-    kc[h * dim + d] = kr[h * dim + d];
+    if (k_norm != nullptr)
+      kc[h * dim + d] = S::from_f32(S::to_f32(kr[h * dim + d]) * k_inv * k_norm[h * dim + d]);
+    else
+      kc[h * dim + d] = kr[h * dim + d];
   }
   const T* vr = v + (int64_t)t * v_stride;
   T* vc = value_cache + slot * (int64_t)kv_heads * vdim;
+  if (v_other != nullptr) {
+    // the cached value is (1 - lambda) v + lambda v_other, v_other another layer's values of this token
+    const float lam = v_blend[0];
+    const T* vo = v_other + (int64_t)t * v_other_stride;
+    for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x)
+      vc[i] = S::from_f32((1.f - lam) * S::to_f32(vr[i]) + lam * S::to_f32(vo[i]));
+    return;
+  }
   if (value_inv_freq == nullptr) {
     for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) vc[i] = vr[i];
     return;
@@ -148,7 +209,7 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void kv_attention_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ token_seq,
     const int64_t* __restrict__ positions, const float* __restrict__ out_inv_freq, int interleaved,
     int heads, int kv_heads, int dim, int vdim, int block_size, int num_blocks, int window,
-    float scale) {
+    float scale, int keep_first, float softcap) {
   __shared__ float q_lds[kHeadsPerGroup][kMaxDim];
   __shared__ float p_lds[kHeadsPerGroup][kWave];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -159,6 +220,9 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void kv_attention_kernel(
   const int p = (int)positions[t];
   const int* table = block_tables + (int64_t)token_seq[t] * max_blocks;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int nk = min(keep_first, lo);         // kept keys ahead of the window
+  const int total = nk + p - lo + 1;
+  auto key_of = [&](int u) { return u < nk ? u : u - nk + lo; };
   for (int d = lane; d < dim; d += kWave)
     q_lds[w][d] = S::to_f32(q[(int64_t)t * q_stride + (int64_t)h * dim + d]) * scale;
   wave_sync();
@@ -173,17 +237,17 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void kv_attention_kernel(
 #pragma unroll
   for (int c = 0; c < kAccum; ++c) acc[c] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int j0 = lo; j0 <= p; j0 += kWave) {
-    const int j = j0 + lane;
+  for (int u0 = 0; u0 < total; u0 += kWave) {
+    const int u = u0 + lane;
     float s = -INFINITY;
-    if (j <= p) {
-      const typename S::T* kr = key_cache + token_row(j) * dim;
+    if (u < total) {
+      const typename S::T* kr = key_cache + token_row(key_of(u)) * dim;
       float dot = 0.f;
       for (int d = 0; d < dim; ++d) dot += q_lds[w][d] * S::to_f32(kr[d]);
-      s = dot;
+      s = softcap > 0.f ? cap_score(dot, softcap) : dot;
     }
     const float m_new = fmaxf(m, wave_max(s));
-    const float pj = j <= p ? expf(s - m_new) : 0.f;
+    const float pj = u < total ? expf(s - m_new) : 0.f;
     const float corr = expf(m - m_new);  // first tile: exp(-inf) = 0
     l = l * corr + wave_sum(pj);
     m = m_new;
@@ -192,9 +256,9 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void kv_attention_kernel(
     wave_sync();
 #pragma unroll
     for (int c = 0; c < kAccum; ++c) acc[c] *= corr;
-    const int n = min(kWave, p - j0 + 1);
+    const int n = min(kWave, total - u0);
     for (int jj = 0; jj < n; ++jj) {
-      const typename S::T* vr = value_cache + token_row(j0 + jj) * vdim;
+      const typename S::T* vr = value_cache + token_row(key_of(u0 + jj)) * vdim;
       const float pv = p_lds[w][jj];
 #pragma unroll
       for (int c = 0; c < kAccum; ++c) {
@@ -363,7 +427,8 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
     const typename S::T* __restrict__ key_cache, const typename S::T* __restrict__ value_cache,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ query_start_loc,
     const int* __restrict__ context_lens, const float* __restrict__ out_inv_freq, int interleaved,
-    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale, int head_waves) {
+    int heads, int kv_heads, int block_size, int num_blocks, int window, float scale, int head_waves,
+    int keep_first, float softcap) {
   using T = typename S::T;
   using M = Mfma16<S>;
   constexpr int D = 32 * DB, VD = 32 * VB;
@@ -395,8 +460,14 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   const int p0 = p_first + kTile * rb;                // this wave's first position
   const int pq = p0 + c;
   const int j_lo = window > 0 ? max(0, p_first - window + 1) : 0;
+  // the keys this workgroup walks, through one index: the kept first tokens that lie ahead of the
+  // first row's window, then the window's first key to the last row
+  const int nk = min(keep_first, j_lo);
+  const int total = nk + p_last - j_lo + 1;
+  auto key_of = [&](int u) { return u < nk ? u : u - nk + j_lo; };
   const int* table = block_tables + (int64_t)b * max_blocks;
   const float scale2 = scale * 1.4426950408889634f;   // scores in base 2
+  const float cap2 = softcap * 1.4426950408889634f, cap_arg = softcap > 0.f ? 2.f * 1.4426950408889634f / softcap : 0.f;
 
   u32x4 qf[D / 16];
 #pragma unroll
@@ -414,17 +485,17 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   float m = -INFINITY, l = 0.f;
 
   // threads 0 .. 63 look the rows of a tile up: the block id is read one step before it is used
-  auto load_block = [&](int j0) {
-    const int j = j0 + tid;
+  auto load_block = [&](int u0) {
+    const int u = u0 + tid;
     int blk = -1;
-    if (j <= p_last) {
-      blk = table[j / block_size];
+    if (u < total) {
+      blk = table[key_of(u) / block_size];
       blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
     }
     return blk;
   };
-  auto store_row = [&](int j0, int blk, int buf) {
-    const int j = j0 + tid;
+  auto store_row = [&](int u0, int blk, int buf) {
+    const int j = key_of(u0 + tid);
     rows_lds[buf][tid] = blk < 0 ? -1 : ((long long)blk * block_size + j % block_size) * kv_heads + g;
   };
   // staging: DB + VB pieces of 16 bytes per thread and tile
@@ -466,8 +537,8 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   // the block ids of tile it + 3 (whose rows go to rows_lds[(it + 1) & 1] during the step).
   int blk_next = -1;
   if (tid < kKeys) {
-    store_row(j_lo, load_block(j_lo), 0);
-    store_row(j_lo + kKeys, load_block(j_lo + kKeys), 1);
+    store_row(0, load_block(0), 0);
+    store_row(kKeys, load_block(kKeys), 1);
   }
   __syncthreads();
   fetch(0);
@@ -475,16 +546,21 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
   fetch(1);
   __syncthreads();                                     // rows_lds[0] is read: tile 2's rows may go there
   if (tid < kKeys) {
-    store_row(j_lo + 2 * kKeys, load_block(j_lo + 2 * kKeys), 0);
-    blk_next = load_block(j_lo + 3 * kKeys);
+    store_row(2 * kKeys, load_block(2 * kKeys), 0);
+    blk_next = load_block(3 * kKeys);
   }
   __syncthreads();
   int it = 0;
-  for (int j0 = j_lo; j0 <= p_last; j0 += kKeys, ++it) {
+  for (int u0 = 0; u0 < total; u0 += kKeys, ++it) {
     const T* k_lds = k_lds2[it & 1];
     const T* v_lds = v_lds2[it & 1];
-    // keys past this wave's last row, or before its first row's window, are none of its business
-    if (active && j0 <= p0 + nq - 1 && !(window > 0 && j0 + kKeys - 1 < p0 - window + 1)) {
+    // a tile with kept tokens ahead of the window concerns every row; of the others, a tile whose
+    // keys lie past this wave's last row, or before its first row's window (and are not kept ones),
+    // is none of its business
+    const bool kept_tile = u0 < nk;
+    const int j0 = u0 - nk + j_lo;            // the tile's first key when it holds window keys only
+    if (active && (kept_tile || (j0 <= p0 + nq - 1 &&
+                                 !(window > 0 && j0 + kKeys - 1 < p0 - window + 1 && j0 >= keep_first)))) {
       f32x16 st[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
@@ -497,16 +573,19 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
         }
       }
       // every key of the tile visible to every row of the wave: no masks
-      const bool full = j0 + kKeys - 1 <= p0 && nq == kTile && (window <= 0 || p0 + kTile - 1 - j0 < window);
+      const bool full = !kept_tile && j0 + kKeys - 1 <= p0 && nq == kTile &&
+                        (window <= 0 || p0 + kTile - 1 - j0 < window);
       float mt = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           float v = st[kb][i] * scale2;
+          if (softcap > 0.f) v = cap_score_fast(st[kb][i] * scale, cap2, cap_arg);
           if (!full) {
-            const int dist = pq - (j0 + 32 * kb + (i & 3) + 8 * (i >> 2) + 4 * hf);
-            const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window);
+            const int j = key_of(u0 + 32 * kb + (i & 3) + 8 * (i >> 2) + 4 * hf);
+            const int dist = pq - j;
+            const bool ok = c < nq && dist >= 0 && (window <= 0 || dist < window || j < keep_first);
             v = ok ? v : -INFINITY;
           }
           st[kb][i] = v;
@@ -555,12 +634,12 @@ __global__ __launch_bounds__(256, 2) void kv_attention_tile_kernel(
           }
         }
     }
-    if (j0 + kKeys <= p_last) land((it + 1) & 1);              // tile it + 1, fetched a step ago
-    if (j0 + 2 * kKeys <= p_last) fetch(it & 1);               // tile it + 2 on its way
-    if (tid < kKeys && j0 + 3 * kKeys <= p_last) {
+    if (u0 + kKeys < total) land((it + 1) & 1);                // tile it + 1, fetched a step ago
+    if (u0 + 2 * kKeys < total) fetch(it & 1);                 // tile it + 2 on its way
+    if (tid < kKeys && u0 + 3 * kKeys < total) {
       // rows of tile it + 3 into the buffer the step before read tile it + 1's from
-      store_row(j0 + 3 * kKeys, blk_next, (it + 1) & 1);
-      blk_next = load_block(j0 + 4 * kKeys);
+      store_row(u0 + 3 * kKeys, blk_next, (it + 1) & 1);
+      blk_next = load_block(u0 + 4 * kKeys);
     }
     __syncthreads();
   }
@@ -597,7 +676,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ token_seq,
     const int64_t* __restrict__ positions, const float* __restrict__ out_inv_freq, int interleaved,
     int heads, int kv_heads, int block_size, int num_blocks, int window, float scale,
-    int merge_heads) {
+    int merge_heads, int keep_first, float softcap) {
   using T = typename S::T;
   using M = Mfma8<S>;
   constexpr int D = 32 * DB, VD = 32 * VB;
@@ -617,6 +696,9 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
   const int p = (int)positions[t];
   const int* table = block_tables + (int64_t)token_seq[t] * max_blocks;
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int nk = min(keep_first, lo);         // kept keys ahead of the window
+  const int total = nk + p - lo + 1;
+  const float cap_arg = softcap > 0.f ? 2.f * 1.4426950408889634f / softcap : 0.f;
   const bool live = c < nh;
   u32x2 qf[D / 8];
 #pragma unroll
@@ -638,10 +720,11 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
   // row numbers round with shuffles.
   constexpr int KP = D / 8, VP = VD / 8;
   u32x2 xk[KP], xv[VP];
-  auto fetch = [&](int j0) {
-    const int jr = j0 + c;
+  auto fetch = [&](int u0) {
+    const int ur = u0 + c;
     long long row = -1;
-    if (jr <= p) {
+    if (ur < total) {
+      const int jr = ur < nk ? ur : ur - nk + lo;
       int blk = table[jr / block_size];
       blk = (unsigned)blk < (unsigned)num_blocks ? blk : 0;
       row = ((long long)blk * block_size + jr % block_size) * kv_heads + g;
@@ -663,8 +746,8 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
       xv[u] = rb >= 0 ? got : u32x2{0u, 0u};
     }
   };
-  fetch(lo + w * kTile);
-  for (int j0 = lo + w * kTile; j0 <= p; j0 += kRowWaves * kTile) {
+  fetch(w * kTile);
+  for (int u0 = w * kTile; u0 < total; u0 += kRowWaves * kTile) {
 #pragma unroll
     for (int u = 0; u < KP; ++u) {
       const int i = lane + kWave * u;
@@ -677,7 +760,7 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
       const int r = i / (VD / 4), v = i % (VD / 4);
       *reinterpret_cast<u32x2*>(v_lds + r * VROW + 4 * v) = xv[u];
     }
-    if (j0 + kRowWaves * kTile <= p) fetch(j0 + kRowWaves * kTile);
+    if (u0 + kRowWaves * kTile < total) fetch(u0 + kRowWaves * kTile);
     wave_sync();
     f32x16 st;
 #pragma unroll
@@ -690,8 +773,10 @@ __global__ __launch_bounds__(64 * kRowWaves) void kv_attention_heads_kernel(
     float mt = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int dist = p - (j0 + (i & 3) + 8 * (i >> 2) + 4 * hf);
-      st[i] = (live && dist >= 0) ? st[i] * scale : -INFINITY;
+      const int u = u0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
+      float v = st[i] * scale;
+      if (softcap > 0.f) v = cap_score_fast(v, softcap, cap_arg);
+      st[i] = (live && u < total) ? v : -INFINITY;
       mt = fmaxf(mt, st[i]);
     }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
@@ -784,7 +869,7 @@ int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
                      const typename S::T* value_cache, const int* block_tables, int max_blocks,
                      const int* token_seq, const int64_t* positions, const float* out_inv_freq,
                      int interleaved, int heads, int kv_heads, int block_size, int num_blocks,
-                     int window, float scale) {
+                     int window, float scale, int keep_first, float softcap) {
   constexpr int D = 32 * DB, VD = 32 * VB;
   const int group = heads / kv_heads;
   const int merge_heads = group < 32 ? group : 32;
@@ -802,7 +887,7 @@ int launch_heads_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
   kv_attention_heads_kernel<S, DB, VB><<<grid, 64 * kRowWaves, lds, stream>>>(
       out, out_stride, q, q_stride, gate, gate_stride, key_cache, value_cache, block_tables,
       max_blocks, token_seq, positions, out_inv_freq, interleaved, heads, kv_heads, block_size,
-      num_blocks, window, scale, merge_heads);
+      num_blocks, window, scale, merge_heads, keep_first, softcap);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
   return VLA_OK;
 }
@@ -814,11 +899,11 @@ int launch_tiles_one(dim3 grid, hipStream_t stream, typename S::T* out, int64_t 
                      const typename S::T* value_cache, const int* block_tables, int max_blocks,
                      const int* qsl, const int* ctx, const float* out_inv_freq, int interleaved,
                      int heads, int kv_heads, int block_size, int num_blocks, int window,
-                     float scale, int head_waves) {
+                     float scale, int head_waves, int keep_first, float softcap) {
   kv_attention_tile_kernel<S, DB, VB><<<grid, 256, 0, stream>>>(
       out, out_stride, q, q_stride, gate, gate_stride, key_cache, value_cache, block_tables,
       max_blocks, qsl, ctx, out_inv_freq, interleaved, heads, kv_heads, block_size, num_blocks,
-      window, scale, head_waves);
+      window, scale, head_waves, keep_first, softcap);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
   return VLA_OK;
 }
@@ -872,13 +957,16 @@ extern "C" int vla_seq_rotary_kv_write(void* q, int64_t q_stride, const void* k,
                                        const float* value_inv_freq, int num_tokens, int heads,
                                        int kv_heads, int dim, int vdim, int rot_dims,
                                        int interleaved, int block_size, int num_blocks, int dtype,
-                                       void* stream) {
+                                       const float* q_norm, const float* k_norm, float norm_eps,
+                                       const void* v_other, int64_t v_other_stride,
+                                       const float* v_blend, void* stream) {
   if (num_tokens == 0) return VLA_OK;
   if (!q || !k || !v || !key_cache || !value_cache || !positions || !slot_mapping || num_tokens < 0 ||
       heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim ||
       (rot_dims & 1) || (rot_dims > 0 && !inv_freq) || block_size <= 0 || num_blocks <= 0 ||
       q_stride < (int64_t)heads * dim || k_stride < (int64_t)kv_heads * dim ||
-      v_stride < (int64_t)kv_heads * vdim)
+      v_stride < (int64_t)kv_heads * vdim ||
+      (v_other && (!v_blend || value_inv_freq || v_other_stride < (int64_t)kv_heads * vdim)))
     return VLA_ERR_ARG;
   return with_dtype(dtype, [&](auto s) {
     using S = decltype(s);
@@ -886,7 +974,8 @@ extern "C" int vla_seq_rotary_kv_write(void* q, int64_t q_stride, const void* k,
     rotary_kv_write_kernel<S><<<num_tokens, 256, 0, (hipStream_t)stream>>>(
         (T*)q, q_stride, (const T*)k, k_stride, (const T*)v, v_stride, (T*)key_cache,
         (T*)value_cache, positions, slot_mapping, inv_freq, value_inv_freq, heads, kv_heads, dim,
-        vdim, rot_dims, interleaved, (int64_t)num_blocks * block_size);
+        vdim, rot_dims, interleaved, (int64_t)num_blocks * block_size, q_norm, k_norm, norm_eps,
+        (const T*)v_other, v_other_stride, v_blend);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
@@ -899,12 +988,13 @@ extern "C" int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q
                                     const float* out_inv_freq, int interleaved, int num_tokens,
                                     int heads, int kv_heads, int dim, int vdim, int block_size,
                                     int num_blocks, int window, float scale, int dtype,
-                                    void* stream) {
+                                    int keep_first, float softcap, void* stream) {
   if (num_tokens == 0) return VLA_OK;
   if (!out || !q || !key_cache || !value_cache || !block_tables || !token_seq || !positions ||
       num_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || block_size <= 0 ||
       num_blocks <= 0 || max_blocks <= 0 || out_stride < (int64_t)heads * vdim ||
-      q_stride < (int64_t)heads * dim || (gate && gate_stride < heads))
+      q_stride < (int64_t)heads * dim || (gate && gate_stride < heads) || keep_first < 0 ||
+      !(softcap >= 0.f))
     return VLA_ERR_ARG;
   if (dim <= 0 || dim > kMaxDim || vdim <= 0 || vdim > kMaxDim) return VLA_ERR_HEAD_SIZE;
   return with_dtype(dtype, [&](auto s) {
@@ -921,7 +1011,8 @@ extern "C" int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q
                                        (const T*)q, q_stride, (const T*)gate, gate_stride,
                                        (const T*)key_cache, (const T*)value_cache, block_tables,
                                        max_blocks, token_seq, positions, out_inv_freq, interleaved,
-                                       heads, kv_heads, block_size, num_blocks, window, scale);
+                                       heads, kv_heads, block_size, num_blocks, window, scale,
+                                       window > 0 ? keep_first : 0, softcap);
         if (rc != VLA_ERR_HEAD_SIZE) return rc;
       }
     }
@@ -929,7 +1020,8 @@ extern "C" int vla_seq_kv_attention(void* out, int64_t out_stride, const void* q
     kv_attention_kernel<S><<<grid, kWave * kHeadsPerGroup, 0, (hipStream_t)stream>>>(
         (T*)out, out_stride, (const T*)q, q_stride, (const T*)gate, gate_stride,
         (const T*)key_cache, (const T*)value_cache, block_tables, max_blocks, token_seq, positions,
-        out_inv_freq, interleaved, heads, kv_heads, dim, vdim, block_size, num_blocks, window, scale);
+        out_inv_freq, interleaved, heads, kv_heads, dim, vdim, block_size, num_blocks, window, scale,
+        window > 0 ? keep_first : 0, softcap);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
@@ -952,8 +1044,11 @@ extern "C" int vla_seq_kv_attention_tiles(
     int64_t gate_stride, const void* key_cache, const void* value_cache, const int* block_tables,
     int max_blocks, const int* query_start_loc, const int* context_lens, const float* out_inv_freq,
     int interleaved, int num_seqs, int max_query_len, int heads, int kv_heads, int dim, int vdim,
-    int block_size, int num_blocks, int window, float scale, int dtype, void* stream) {
+    int block_size, int num_blocks, int window, float scale, int dtype, int keep_first,
+    float softcap, void* stream) {
   if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
+  if (keep_first < 0 || !(softcap >= 0.f)) return VLA_ERR_ARG;
+  if (window <= 0) keep_first = 0;
   if (!out || !q || !key_cache || !value_cache || !block_tables || !query_start_loc || !context_lens ||
       num_seqs < 0 || num_seqs > 65535 || max_query_len < 0 || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads != 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0 ||
@@ -979,10 +1074,12 @@ extern "C" int vla_seq_kv_attention_tiles(
                               (const __bf16*)q, q_stride, (const __bf16*)gate, gate_stride,
                               (const __bf16*)key_cache, (const __bf16*)value_cache, block_tables,
                               max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved,
-                              heads, kv_heads, block_size, num_blocks, window, scale, head_waves);
+                              heads, kv_heads, block_size, num_blocks, window, scale, head_waves,
+                              keep_first, softcap);
   return launch_tiles<F16>(dim / 32, vdim / 32, grid, (hipStream_t)stream, (_Float16*)out, out_stride,
                            (const _Float16*)q, q_stride, (const _Float16*)gate, gate_stride,
                            (const _Float16*)key_cache, (const _Float16*)value_cache, block_tables,
                            max_blocks, query_start_loc, context_lens, out_inv_freq, interleaved, heads,
-                           kv_heads, block_size, num_blocks, window, scale, head_waves);
+                           kv_heads, block_size, num_blocks, window, scale, head_waves, keep_first,
+                           softcap);
 }

@@ -6,10 +6,13 @@
 //   score = (q_lat,h . c + q_rot,h . k_rot) * scale,    o_lat,h = sum_j p_j c_j,
 // and the head's output is W_uv,h o_lat,h (the caller's product again): every head reads the same
 // rows, nothing per head is cached.  latent_rotary_write norms the step's latents, rotates the
-// shared key part and the queries' rotated parts (interleaved pairs, frequencies from a table, sine
-// and cosine times a magnitude), and writes the cache rows; the attention kernels then read every
-// query row's keys from the cache, so prompts, portions of prompts and decode steps are one case.
-// Angles, norms, scores, softmax and the weighted sum are fp32.
+// shared key part and the queries' rotated parts (pairs (2i, 2i + 1) or (i, i + rot_dims / 2),
+// frequencies from a table, sine and cosine times a magnitude), and writes the cache rows; the
+// attention kernels then read every query row's keys from the cache, so prompts, portions of
+// prompts and decode steps are one case.  An optional window keeps 0 <= p - j < window; an optional
+// gate multiplies a head's sums by the sigmoid of one number per (token, head) (the head's
+// up-projection that follows is linear, so the gate may stand on either side of it).  Angles, norms,
+// scores, softmax and the weighted sum are fp32.
 //
 // latent_attention_kernel: one wave per (token, head), any dtype, rank up to 1024.  A tile is 64
 // keys: lane j scores key j against the query held in LDS, the wave reduces max / sum (online
@@ -43,20 +46,21 @@ __global__ __launch_bounds__(256) void latent_rotary_write_kernel(
     const typename S::T* __restrict__ kv, int64_t kv_stride, const float* __restrict__ norm_weight,
     float eps, typename S::T* __restrict__ cache, const int64_t* __restrict__ positions,
     const int64_t* __restrict__ slot_mapping, const float* __restrict__ inv_freq, float magnitude,
-    int heads, int rank, int rot, int rot_dims, int64_t num_slots) {
+    int heads, int rank, int rot, int rot_dims, int64_t num_slots, int interleaved) {
   using T = typename S::T;
   __shared__ float red[16];
   const int t = blockIdx.x;
   const float p = (float)positions[t];
   const int half = rot_dims / 2;        // pairs that turn; what follows them passes unchanged
+  const int first_mul = interleaved ? 2 : 1, second = interleaved ? 1 : half;   // pair f: f * first_mul, + second
   T* qr = q + (int64_t)t * q_stride + q_first;
   for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
     const int h = i / half, f = i - h * half;
-    T* e = qr + (int64_t)h * q_head_stride + 2 * f;
-    float a = S::to_f32(e[0]), b = S::to_f32(e[1]);
+    T* e = qr + (int64_t)h * q_head_stride + first_mul * f;
+    float a = S::to_f32(e[0]), b = S::to_f32(e[second]);
     turn_scaled(a, b, p * inv_freq[f], magnitude);
     e[0] = S::from_f32(a);
-    e[1] = S::from_f32(b);
+    e[second] = S::from_f32(b);
   }
   const int64_t slot = slot_mapping[t];
   const bool cached = slot >= 0 && slot < num_slots;    // uniform over the workgroup
@@ -73,10 +77,10 @@ __global__ __launch_bounds__(256) void latent_rotary_write_kernel(
   for (int c = threadIdx.x; c < rank; c += blockDim.x)
     row[c] = S::from_f32(S::to_f32(kr[c]) * inv * norm_weight[c]);
   for (int f = threadIdx.x; f < half; f += blockDim.x) {
-    float a = S::to_f32(kr[rank + 2 * f]), b = S::to_f32(kr[rank + 2 * f + 1]);
+    float a = S::to_f32(kr[rank + first_mul * f]), b = S::to_f32(kr[rank + first_mul * f + second]);
     turn_scaled(a, b, p * inv_freq[f], magnitude);
-    row[rank + 2 * f] = S::from_f32(a);
-    row[rank + 2 * f + 1] = S::from_f32(b);
+    row[rank + first_mul * f] = S::from_f32(a);
+    row[rank + first_mul * f + second] = S::from_f32(b);
   }
   for (int c = 2 * half + threadIdx.x; c < rot; c += blockDim.x) row[rank + c] = kr[rank + c];
 }
@@ -94,7 +98,8 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
     typename S::T* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride,
     LatentQuery<S> q, const typename S::T* __restrict__ cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
-    int heads, int rank, int rot, int block_size, int num_blocks, float scale) {
+    int heads, int rank, int rot, int block_size, int num_blocks, float scale, int window,
+    const typename S::T* __restrict__ gate, int64_t gate_stride) {
   extern __shared__ float lds[];
   const int width = rank + rot;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -121,7 +126,8 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
 #pragma unroll
   for (int c = 0; c < kAccum; ++c) acc[c] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int j0 = 0; j0 <= p; j0 += kWave) {
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  for (int j0 = lo; j0 <= p; j0 += kWave) {
     const int j = j0 + lane;
     float s = -INFINITY;
     if (j <= p) {
@@ -151,7 +157,8 @@ __global__ __launch_bounds__(kWave* kHeadsPerGroup) void latent_attention_kernel
       }
     }
   }
-  const float inv = 1.f / l;
+  float inv = 1.f / l;
+  if (gate != nullptr) inv /= 1.f + expf(-S::to_f32(gate[(int64_t)t * gate_stride + h]));
   typename S::T* orow = out + (int64_t)t * out_token_stride + (int64_t)h * out_head_stride;
 #pragma unroll
   for (int c = 0; c < kAccum; ++c) {
@@ -218,7 +225,8 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     LatentQuery<S> q, const typename S::T* __restrict__ cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
     int heads, int rank, int rot, int block_size, int num_blocks, float scale, int hb, int tb,
-    int key_splits, float* __restrict__ part_o, float* __restrict__ part_ml, int num_tokens) {
+    int key_splits, float* __restrict__ part_o, float* __restrict__ part_ml, int num_tokens,
+    int window, const typename S::T* __restrict__ gate, int64_t gate_stride) {
   using T = typename S::T;
   using M = LatentMfma<S>;
   constexpr int WP = 2 * VBW + 2;                      // 16-byte pieces of a tile a thread stages
@@ -241,9 +249,11 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
   const int hf = lane >> 5, c = lane & 31;
   const int t_first = query_start_loc[b] + tq0;
   const int p_first = context_lens[b] + tq0, p_end = p_first + ntok - 1;
-  // this workgroup's share of the keys 0 .. p_end: whole tiles, the last share may be short or empty
-  const int share = ((p_end + key_splits) / key_splits + kTileKeys - 1) / kTileKeys * kTileKeys;
-  const int j_begin = split * share;
+  // this workgroup's share of the keys j_first .. p_end (j_first: where the first row's window
+  // starts): whole tiles, the last share may be short or empty
+  const int j_first = window > 0 ? max(0, p_first - window + 1) : 0;
+  const int share = ((p_end - j_first + key_splits) / key_splits + kTileKeys - 1) / kTileKeys * kTileKeys;
+  const int j_begin = j_first + split * share;
   const int p_last = min(p_end, j_begin + share - 1);      // the last key this workgroup reads
   const int my_tok = c / hb, my_head = c - my_tok * hb;
   const bool my_row = my_tok < ntok && my_head < nh;
@@ -367,14 +377,14 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     // (the sum above runs in a different order in each wave; every wave keeps its own max and sum, and
     // they only need to agree with its own weights)
     // every key of the tile visible to every row of a full workgroup: no masks
-    const bool full = all_rows && j0 + kTileKeys - 1 <= p_first;
+    const bool full = all_rows && j0 + kTileKeys - 1 <= p_first && (window <= 0 || p_end - j0 < window);
     float mt = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       float v = st[i] * scale2;
       if (!full) {
         const int j = j0 + (i & 3) + 8 * (i >> 2) + 4 * hf;
-        v = my_row && j <= pq ? v : -INFINITY;
+        v = my_row && j <= pq && (window <= 0 || pq - j < window) ? v : -INFINITY;
       }
       st[i] = v;
       mt = fmaxf(mt, v);
@@ -447,7 +457,8 @@ __global__ __launch_bounds__(256) void latent_attention_tile_kernel(
     }
     return;
   }
-  const float inv = 1.f / l;
+  float inv = 1.f / l;
+  if (gate != nullptr) inv /= 1.f + expf(-S::to_f32(gate[(int64_t)(t_first + my_tok) * gate_stride + h0 + my_head]));
   T* orow = out + (int64_t)(t_first + my_tok) * out_token_stride + (int64_t)(h0 + my_head) * out_head_stride;
 #pragma unroll
   for (int n = 0; n < VBW; ++n) {
@@ -466,10 +477,11 @@ template <class S>
 __global__ __launch_bounds__(256) void latent_merge_kernel(
     typename S::T* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride,
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int key_splits,
-    int num_tokens, int heads, int rank) {
+    int num_tokens, int heads, int rank, const typename S::T* __restrict__ gate, int64_t gate_stride) {
   const int64_t th = blockIdx.x;                 // token * heads + head
   const int64_t t = th / heads;
   const int h = (int)(th - t * heads);
+  const float gv = gate != nullptr ? 1.f / (1.f + expf(-S::to_f32(gate[t * gate_stride + h]))) : 1.f;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     const int w = (d >> 5) & 3;
     const int64_t stride = (int64_t)num_tokens * heads;        // rows between two shares
@@ -486,7 +498,7 @@ __global__ __launch_bounds__(256) void latent_merge_kernel(
       num += ov * f;
       den += ls * f;
     }
-    out[t * out_token_stride + h * out_head_stride + d] = S::from_f32(num / den);
+    out[t * out_token_stride + h * out_head_stride + d] = S::from_f32(num / den * gv);
   }
 }
 
@@ -504,7 +516,8 @@ int launch_latent_tiles(dim3 grid, size_t lds, hipStream_t stream, typename S::T
                         const typename S::T* cache, const int* block_tables, int max_blocks,
                         const int* qsl, const int* ctx, int heads, int rank, int rot, int block_size,
                         int num_blocks, float scale, int hb, int tb, int key_splits, float* part_o,
-                        float* part_ml, int num_tokens) {
+                        float* part_ml, int num_tokens, int window, const typename S::T* gate,
+                        int64_t gate_stride) {
   static std::atomic<size_t> allowed{64 * 1024};   // raised once per kernel, not per launch
   if (lds > allowed.load(std::memory_order_relaxed)) {
     VLA_SEQ_HIP_CHECK(hipFuncSetAttribute(
@@ -514,11 +527,13 @@ int launch_latent_tiles(dim3 grid, size_t lds, hipStream_t stream, typename S::T
   }
   latent_attention_tile_kernel<S, VBW><<<grid, 256, lds, stream>>>(
       out, out_token_stride, out_head_stride, q, cache, block_tables, max_blocks, qsl, ctx, heads,
-      rank, rot, block_size, num_blocks, scale, hb, tb, key_splits, part_o, part_ml, num_tokens);
+      rank, rot, block_size, num_blocks, scale, hb, tb, key_splits, part_o, part_ml, num_tokens,
+      window, gate, gate_stride);
   VLA_SEQ_HIP_CHECK(hipGetLastError());
   if (key_splits > 1) {
     latent_merge_kernel<S><<<(unsigned)((int64_t)num_tokens * heads), 256, 0, stream>>>(
-        out, out_token_stride, out_head_stride, part_o, part_ml, key_splits, num_tokens, heads, rank);
+        out, out_token_stride, out_head_stride, part_o, part_ml, key_splits, num_tokens, heads, rank,
+        gate, gate_stride);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
   }
   return VLA_OK;
@@ -538,7 +553,7 @@ extern "C" int vla_seq_latent_rotary_write(void* q, int64_t q_stride, int q_head
                                            const float* inv_freq, float magnitude, int num_tokens,
                                            int heads, int rank, int rot, int rot_dims,
                                            int block_size, int num_blocks, int dtype,
-                                           void* stream) {
+                                           int interleaved, void* stream) {
   if (num_tokens == 0) return VLA_OK;
   if (!q || !kv || !norm_weight || !cache || !positions || !slot_mapping || num_tokens < 0 ||
       heads <= 0 || rank <= 0 || rot < 0 || rot_dims < 0 || rot_dims > rot || (rot_dims & 1) ||
@@ -552,7 +567,7 @@ extern "C" int vla_seq_latent_rotary_write(void* q, int64_t q_stride, int q_head
     latent_rotary_write_kernel<S><<<num_tokens, 256, 0, (hipStream_t)stream>>>(
         (T*)q, q_stride, q_head_stride, q_first, (const T*)kv, kv_stride, norm_weight, eps, (T*)cache,
         positions, slot_mapping, inv_freq, magnitude, heads, rank, rot, rot_dims,
-        (int64_t)num_blocks * block_size);
+        (int64_t)num_blocks * block_size, interleaved);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
@@ -565,8 +580,10 @@ extern "C" int vla_seq_latent_attention(void* out, int64_t out_token_stride, int
                                         const void* cache, const int* block_tables, int max_blocks,
                                         const int* token_seq, const int64_t* positions,
                                         int num_tokens, int heads, int rank, int rot, int block_size,
-                                        int num_blocks, float scale, int dtype, void* stream) {
+                                        int num_blocks, float scale, int dtype, int window,
+                                        const void* gate, int64_t gate_stride, void* stream) {
   if (num_tokens == 0) return VLA_OK;
+  if (gate && gate_stride < heads) return VLA_ERR_ARG;
   if (!out || !q_lat || (rot > 0 && !q_rot) || !cache || !block_tables || !token_seq || !positions ||
       num_tokens < 0 || heads <= 0 || rot < 0 || block_size <= 0 || num_blocks <= 0 ||
       max_blocks <= 0)
@@ -581,7 +598,8 @@ extern "C" int vla_seq_latent_attention(void* out, int64_t out_token_stride, int
     const size_t lds = (size_t)kHeadsPerGroup * (rank + rot + kWave) * sizeof(float);
     latent_attention_kernel<S><<<grid, kWave * kHeadsPerGroup, lds, (hipStream_t)stream>>>(
         (T*)out, out_token_stride, out_head_stride, q, (const T*)cache, block_tables, max_blocks,
-        token_seq, positions, heads, rank, rot, block_size, num_blocks, scale);
+        token_seq, positions, heads, rank, rot, block_size, num_blocks, scale, window, (const T*)gate,
+        gate_stride);
     VLA_SEQ_HIP_CHECK(hipGetLastError());
     return VLA_OK;
   });
@@ -610,8 +628,9 @@ extern "C" int vla_seq_latent_attention_tiles(
     int64_t rot_head_stride, const void* cache, const int* block_tables, int max_blocks,
     const int* query_start_loc, const int* context_lens, int num_seqs, int max_query_len, int heads,
     int rank, int rot, int block_size, int num_blocks, float scale, int key_splits, float* scratch,
-    int num_tokens, int dtype, void* stream) {
+    int num_tokens, int dtype, int window, const void* gate, int64_t gate_stride, void* stream) {
   if (num_seqs == 0 || max_query_len == 0) return VLA_OK;
+  if (gate && gate_stride < heads) return VLA_ERR_ARG;
   if (!out || !q_lat || (rot > 0 && !q_rot) || !cache || !block_tables || !query_start_loc ||
       !context_lens || num_seqs < 0 || num_seqs > 65535 || max_query_len < 0 || heads <= 0 ||
       rot < 0 || block_size <= 0 || num_blocks <= 0 || max_blocks <= 0 || key_splits < 1 ||
@@ -644,7 +663,7 @@ extern "C" int vla_seq_latent_attention_tiles(
                                      out_head_stride, q, (const T*)cache, block_tables, max_blocks, \
                                      query_start_loc, context_lens, heads, rank, rot, block_size,   \
                                      num_blocks, scale, hb, tb, key_splits, part_o, part_ml,        \
-                                     num_tokens);
+                                     num_tokens, window, (const T*)gate, gate_stride);
     switch (vbw) {
       VLA_LATENT_CASE(1)
       VLA_LATENT_CASE(2)

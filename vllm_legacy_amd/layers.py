@@ -218,16 +218,55 @@ class TokenGatedInput(nn.Module):
 
 class GatedActivation(nn.Module):
     """act(gate) * up on the two halves of a merged projection [T, 2 F] (gate | up), or act(z) on
-    a plain one; act: relu, relu2 (the square of relu), silu, gelu_tanh."""
+    a plain one; act: relu, relu2 (the square of relu), silu, gelu_tanh.  The gated form
+    "clamped_glu" is g sigmoid(alpha g) (u + shift) with g = min(gate, limit) and
+    u = clamp(up, -limit, limit)."""
 
-    def __init__(self, act: str, gated: bool = True):
+    def __init__(self, act: str, gated: bool = True, limit: float = 0.0, alpha: float = 1.702, shift: float = 1.0):
         super().__init__()
-        if act not in seq_ops.ACT or act == "none":
+        if act == "clamped_glu":
+            if not (gated and limit > 0):
+                raise ValueError("clamped_glu is a gated activation with a positive limit")
+        elif act not in seq_ops.ACT or act == "none":
             raise ValueError(f"unknown activation {act!r}")
         self.act, self.gated = act, gated
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
 
     def forward(self, z: torch.Tensor) -> torch.Tensor:
         F = z.shape[1] // 2 if self.gated else z.shape[1]
         out = torch.empty((z.shape[0], F), dtype=z.dtype, device=z.device)
-        seq_ops.gated_act(out, z[:, :F], z[:, F:] if self.gated else None, self.act)
+        if self.act == "clamped_glu":
+            seq_ops.clamped_glu(out, z[:, :F], z[:, F:], self.limit, self.alpha, self.shift)
+        else:
+            seq_ops.gated_act(out, z[:, :F], z[:, F:] if self.gated else None, self.act)
+        return out
+
+
+class PairHashEmbedding(nn.Module):
+    """Token embedding plus a hashed embedding of the (previous token, token) pair, written as the
+    fp32 stream: row (prev * mul_prev + token * mul_cur) mod buckets of a second table, its last row
+    (number `buckets`) for a sequence's first token.  A sequence's last token lives in a state slot
+    (int64 [num_slots]) between steps, so a sequence may be cut anywhere."""
+
+    def __init__(self, vocab_size: int, width: int, buckets: int, mul_prev: int, mul_cur: int,
+                 dtype=torch.bfloat16, device=None):
+        super().__init__()
+        if buckets < 1 or mul_prev < 0 or mul_cur < 0:
+            raise ValueError("buckets must be positive and the multipliers non-negative")
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.weight = nn.Parameter(torch.zeros((vocab_size, width), dtype=dtype, device=device),
+                                   requires_grad=False)
+        self.pair_weight = nn.Parameter(torch.zeros((buckets + 1, width), dtype=dtype, device=device),
+                                        requires_grad=False)
+
+    @staticmethod
+    def get_state_shape(num_slots: int) -> Tuple[int, ...]:
+        return (num_slots, )
+
+    def forward(self, input_ids: torch.Tensor, last_token: torch.Tensor, batch) -> torch.Tensor:
+        out = torch.empty((input_ids.numel(), self.weight.shape[1]), dtype=torch.float32,
+                          device=self.weight.device)
+        seq_ops.pair_hash_embed(out, self.weight.data, self.pair_weight.data, input_ids, last_token,
+                                batch.query_start_loc, batch.context_lens, batch.state_slots, batch.token_seq,
+                                self.mul_prev, self.mul_cur)
         return out

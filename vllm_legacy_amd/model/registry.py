@@ -13,6 +13,7 @@ _MODELS: Dict[str, Tuple[str, str, str]] = {
     "Lusadra": ("vllm_legacy_amd.model.lusadra", "LusadraForCausalLM", "LusadraConfig"),
     "Dopipel": ("vllm_legacy_amd.model.dopipel", "DopipelForCausalLM", "DopipelConfig"),
     "Lamosun": ("vllm_legacy_amd.model.lamosun", "LamosunForCausalLM", "LamosunConfig"),
+    "Tekezen": ("vllm_legacy_amd.model.tekezen", "TekezenForCausalLM", "TekezenConfig"),
     # the synthetic-weight Llama stack behind the engine's model protocol
     "LlamaDecodeStack": ("vllm_legacy_amd.engine.llama_adapter", "PagedLlamaForEngine", "LlamaEngineConfig"),
 }

@@ -4,8 +4,11 @@ Router: z = W_r h (+ a bias) in fp32 over all routed experts, s = softmax(z); th
 with the largest s + correction are chosen and weighted by their s renormalized to sum 1 (without a
 correction: the softmax over the chosen logits).  The last `identity` routed experts have no
 weights: their output is the token's input.  An expert is W_down act(W_up h), or, `gated`,
-W_down (act(W_gate h) * W_up h).  An optional shared expert of the same form runs for every token, multiplied by
-sigmoid(w_sg . h).  The output is fp32 (the caller norms it and adds it to its stream).
+W_down (act(W_gate h) * W_up h); with act "clamped_glu" the gated form is
+g sigmoid(alpha g) (u + shift), g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit).  An
+optional shared expert runs for every token: plain, multiplied by sigmoid(w_sg . h), or
+(`shared_gated`) of the gated form with a limit of its own and nothing in front.  The output is
+fp32 (the caller norms it and adds it to its stream).
 
 Execution (csrc/seq_moe_kernels.hip): route (the logits of a large step come from one fp32 matrix
 product) -> plan (pairs grouped by expert into row tiles) ->
@@ -35,8 +38,16 @@ class RoutedExperts(nn.Module):
 
     def __init__(self, width: int, num_experts: int, num_identity: int, top: int, expert_ff: int,
                  shared_ff: int = 0, act: str = "relu2", shared_act: Optional[str] = None,
-                 dtype=torch.bfloat16, device=None, gated: bool = False, router_bias: bool = False) -> None:
+                 dtype=torch.bfloat16, device=None, gated: bool = False, router_bias: bool = False,
+                 act_limit: float = 0.0, act_alpha: float = 1.702, act_shift: float = 1.0,
+                 shared_gated: bool = False, shared_limit: float = 0.0) -> None:
         super().__init__()
+        if act == "clamped_glu" and not (gated and act_limit > 0):
+            raise ValueError("clamped_glu needs gated experts and a limit")
+        if shared_gated and shared_ff and (shared_act or act) == "clamped_glu" and not shared_limit > 0:
+            raise ValueError("a clamped_glu shared expert needs a limit")
+        self.act_limit, self.act_alpha, self.act_shift = float(act_limit), float(act_alpha), float(act_shift)
+        self.shared_gated, self.shared_limit = bool(shared_gated), float(shared_limit)
         if top > num_experts + num_identity:
             raise ValueError("top exceeds the number of routed experts")
         self.width, self.num_experts, self.num_identity, self.top = width, num_experts, num_identity, top
@@ -57,13 +68,14 @@ class RoutedExperts(nn.Module):
         self.w_up = par((num_experts, (2 if gated else 1) * expert_ff, width), dtype)
         self.w_down = par((num_experts, width, expert_ff), dtype)
         if shared_ff:
-            self.shared_up = par((shared_ff, width), dtype)
+            # a gated shared expert keeps W_gate's rows ahead of W_up's and has no sigmoid in front
+            self.shared_up = par(((2 if shared_gated else 1) * shared_ff, width), dtype)
             self.shared_down = par((width, shared_ff), dtype)
-            self.shared_gate = par((width, ), torch.float32)
+            self.shared_gate = None if shared_gated else par((width, ), torch.float32)
 
     def set_weights(self, t: Dict[str, torch.Tensor]) -> None:
         """t: router, router.b (with a router bias), correction (optional), e<i>.up / e<i>.down
-        (gated: also e<i>.gate), shared.up / shared.down / shared.sg."""
+        (gated: also e<i>.gate), shared.up / shared.down and shared.sg or (gated) shared.gate."""
         dev, dt = self.router.device, self.dtype
         routed = self.num_experts + self.num_identity
 
@@ -86,16 +98,25 @@ class RoutedExperts(nn.Module):
         if self.num_experts:
             put(self.w_down, torch.stack([t[f"e{e}.down"] for e in range(self.num_experts)]).to(dt), "e*.down")
         if self.shared_ff:
-            put(self.shared_up, t["shared.up"], "shared.up")
+            if self.shared_gated:
+                put(self.shared_up, torch.cat([t["shared.gate"], t["shared.up"]], 0), "shared.gate | shared.up")
+            else:
+                put(self.shared_up, t["shared.up"], "shared.up")
+                put(self.shared_gate, t["shared.sg"].reshape(self.width), "shared.sg")
             put(self.shared_down, t["shared.down"], "shared.down")
-            put(self.shared_gate, t["shared.sg"].reshape(self.width), "shared.sg")
 
     def router_rows(self) -> torch.Tensor:
         """fp32 [routed (+ 1), width]: the router and, last, the shared expert's gate."""
         if self._router_rows is None:
             self._router_rows = torch.cat([self.router.data, self.shared_gate.data[None]], 0).contiguous() \
-                if self.shared_ff else self.router.data
+                if self.shared_gate is not None else self.router.data
         return self._router_rows
+
+    def _glu(self, out: torch.Tensor, both: torch.Tensor, ff: int, act: str, limit: float) -> None:
+        if act == "clamped_glu":
+            ops.clamped_glu(out, both[:, :ff], both[:, ff:], limit, self.act_alpha, self.act_shift)
+        else:
+            ops.gated_act(out, both[:, :ff], both[:, ff:], act)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         """h [T, width] in the activation dtype -> fp32 [T, width]."""
@@ -105,7 +126,7 @@ class RoutedExperts(nn.Module):
             # many tokens: the router rows (and the shared gate's) as one fp32 matrix product
             logits = torch.mm(h if h.dtype == torch.float32 else h.float(), self.router_rows().t())
         experts, weights, sg = ops.moe_route(h, self.router.data, self.correction.data,
-                                             self.shared_gate.data if self.shared_ff else None, self.top, logits,
+                                             None if self.shared_gate is None else self.shared_gate.data, self.top, logits,
                                              None if self.router_bias is None else self.router_bias.data)
         if self.num_experts:
             pair_row, row_token, tile_expert = ops.moe_plan(experts, self.num_experts)
@@ -114,7 +135,7 @@ class RoutedExperts(nn.Module):
             if self.gated:
                 both = torch.empty((rows, 2 * self.expert_ff), dtype=h.dtype, device=h.device)
                 ops.grouped_linear(both, h, row_token, self.w_up.data, tile_expert)
-                ops.gated_act(u, both[:, :self.expert_ff], both[:, self.expert_ff:], self.act)
+                self._glu(u, both, self.expert_ff, self.act, self.act_limit)
             else:
                 ops.grouped_linear(u, h, row_token, self.w_up.data, tile_expert, self.act)
             y = torch.empty((rows, self.width), dtype=torch.float32, device=h.device)
@@ -125,8 +146,12 @@ class RoutedExperts(nn.Module):
         shared_y = None
         if self.shared_ff:
             su = torch.mm(h, self.shared_up.data.t())
-            sa = torch.empty_like(su)
-            ops.gated_act(sa, su, None, self.shared_act)
+            if self.shared_gated:
+                sa = torch.empty((T, self.shared_ff), dtype=su.dtype, device=su.device)
+                self._glu(sa, su, self.shared_ff, self.shared_act, self.shared_limit)
+            else:
+                sa = torch.empty_like(su)
+                ops.gated_act(sa, su, None, self.shared_act)
             shared_y = mm_f32(sa, self.shared_down.data)
         out = torch.empty((T, self.width), dtype=torch.float32, device=h.device)
         ops.moe_combine(out, y, pair_row, weights, h, shared_y, sg)
