@@ -67,6 +67,7 @@ class RoutedExperts(nn.Module):
         # gated experts keep W_gate's rows ahead of W_up's in one matrix per expert
         self.w_up = par((num_experts, (2 if gated else 1) * expert_ff, width), dtype)
         self.w_down = par((num_experts, width, expert_ff), dtype)
+        self.shared_gate = None
         if shared_ff:
             # a gated shared expert keeps W_gate's rows ahead of W_up's and has no sigmoid in front
             self.shared_up = par(((2 if shared_gated else 1) * shared_ff, width), dtype)
