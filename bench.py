@@ -55,11 +55,11 @@ def parse():
     ap.add_argument("--rank-of", type=int, default=1,
                     help="kernel study: one process with the per-GPU shapes of an N-way tensor-"
                          "parallel rank (heads, FFN and vocabulary divided by N, no collectives)")
-    ap.add_argument("--arch", default=None, choices=["lusadra", "dopipel", "lamosun"],
+    ap.add_argument("--arch", default=None, choices=["lusadra", "dopipel", "lamosun", "tekezen"],
                     help="instead of the decode-step benchmark: prefill / decode throughput of this "
                          "architecture beside the Llama stack at equal size, and its kernels beside "
                          "the like kernels against their rooflines (tools/seq_arch_bench.py, tools/dopipel_bench.py, "
-                         "tools/lamosun_bench.py; lamosun stands beside Dopipel)")
+                         "tools/lamosun_bench.py, tools/tekezen_bench.py; lamosun and tekezen stand beside Dopipel)")
     ap.add_argument("--arch-size", default="2k", choices=["2k", "4k"])
     ap.add_argument("--arch-prompt", type=int, default=4096)
     ap.add_argument("--arch-batch", type=int, default=64)
@@ -342,6 +342,9 @@ def main():
         elif args.arch == "lamosun":
             from tools import lamosun_bench
             lamosun_bench.run(args)
+        elif args.arch == "tekezen":
+            from tools import tekezen_bench
+            tekezen_bench.run(args)
         else:
             from tools import seq_arch_bench
             seq_arch_bench.run(args)
