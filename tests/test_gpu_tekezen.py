@@ -63,6 +63,13 @@ def configs():
                                 A(2, 1, 8, window=500, keep_first=4, factor=8.0, v_mix=True, mlp=M(20, 3.0)),
                                 L(3, 8, 4, 8, 12, window=500, scaling=YARN, mlp=M(24))], width=48, buckets=997,
                                mul_prev=1000003, mul_cur=999983),
+        # nothing a multiple of four: widths, ranks, head sizes, vocabulary, feed-forward sizes
+        "ragged": R.make_config([
+            A(3, 3, 10, vdim=14, window=11, keep_first=2, rot_dims=6, factor=2.5, softcap=9.0, mlp=E(5, 2, 18, 2.0, 6, 1.0)),
+            L(3, 10, 6, 14, 18, window=7, scaling=YARN, mlp=M(50)),
+            A(1, 1, 22, vdim=42, window=5, keep_first=1, rot_dims=2, v_mix=True, mlp=E(4, 4, 6, 1.0)),
+            A(6, 1, 6, vdim=42, window=30, rot_dims=6, v_mix=True, mlp=None)],
+            vocab=101, width=50, buckets=11, mul_prev=2, mul_cur=9),
         # sizes for the matrix-core kernels: multiples of 32, many heads
         "mfma": R.make_config([
             A(8, 2, 32, vdim=64, window=20, keep_first=4, rot_dims=16, factor=2.0, softcap=15.0, v_mix=True, mlp=M(64)),
@@ -300,6 +307,8 @@ ATTN_SHAPES = [
     (8, 1, 64, 32, 32, 64, 6, 0.0, 4.0),
     (5, 5, 128, 128, 64, 17, 40, 30.0, 2.0),
     (4, 2, 32, 96, 32, 0, 0, 6.0, 1.0),
+    (6, 2, 64, 32, 16, 60, 5, 18.0, 3.0),
+    (4, 1, 32, 32, 16, 10, 3, 0.0, 1.0),
 ]
 
 
@@ -606,7 +615,7 @@ def test_whole_prompt_portions_and_decoding_agree_with_the_reference(tmp_path, n
         within(logit_error(run(sizes, sid), want), dtype, sid)
 
 
-@pytest.mark.parametrize("name", ["plain", "odd", "equal", "edges"])
+@pytest.mark.parametrize("name", ["plain", "odd", "equal", "edges", "ragged"])
 def test_layer_by_layer_against_the_reference(tmp_path, name):
     """The stream after every layer, float32."""
     s = Served(tmp_path, name, torch.float32)
